@@ -1,0 +1,81 @@
+"""ctypes binding of libdcp_hip.so.
+
+The library is the only compute backend: if it is missing or fails to load,
+every operator raises instead of falling back to another implementation.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libdcp_hip.so"
+
+_P = c_void_p
+_I = c_int
+_L = c_int64
+_F = c_float
+
+# symbol -> argument types (all return int unless noted)
+SIGNATURES = {
+    "dcp_version": [],
+    "dcp_last_error": [],
+    "dcp_fused_copy_varlen": [_P, _P, _P, _P, _P, _P, _P, _I, _L, _I, _P],
+    "dcp_fused_copy_varlen_dkv": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "dcp_fused_copy_varlen_lse": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "dcp_update_out_lse": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _L, _L, _L, _L, _L, _L, _I, _I, _I, _P],
+    "dcp_blockwise_sum": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _P],
+    "dcp_attn_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _F, _I, _P],
+    "dcp_attn_bwd": [_P] * 14 + [_I] + [_P] * 5 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class DcpHipError(RuntimeError):
+    """The HIP library is unavailable or rejected a call."""
+
+
+def load():
+    """Return the loaded library (loads it on first use)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise DcpHipError(
+                f"{LIB_PATH} is not built; run `python -m dcp_amd.build` "
+                "(there is no fallback implementation)"
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = c_char_p if name == "dcp_last_error" else c_int
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().dcp_last_error().decode(errors="replace")
+
+
+def call(name: str, *args) -> None:
+    """Call an entry point; a nonzero status becomes an exception carrying the
+    library's message: ``ValueError`` for unsupported types (status 2),
+    ``AssertionError`` for argument preconditions (status 1), as the reference
+    operators raise for the same conditions."""
+    status = getattr(load(), name)(*args)
+    if status == 0:
+        return
+    message = f"{name}: {last_error()}"
+    if status == 2:
+        raise ValueError(message)
+    if status == 1:
+        raise AssertionError(message)
+    raise DcpHipError(message)

@@ -1,0 +1,70 @@
+"""Builds libdcp_hip.so (the C-ABI kernel library) in-tree with hipcc.
+
+``python -m dcp_amd.build`` compiles every source under ``dcp_amd/csrc`` for
+gfx950 and links ``dcp_amd/libdcp_hip.so``.  hipcc cross-compiles, so no GPU is
+needed to build.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+INCLUDE = PKG_DIR.parent / "include"
+LIB_PATH = PKG_DIR / "libdcp_hip.so"
+BUILD_DIR = PKG_DIR / "csrc" / "build"
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Wno-unused-value",
+    f"-I{INCLUDE}",
+    f"-I{CSRC}",
+    # keep the compiler from forming packed-fp32 VALU ops
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+]
+
+
+def sources():
+    return sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
+
+
+def _compile(src: Path) -> Path:
+    obj = BUILD_DIR / (src.name + ".o")
+    lang = ["-x", "hip"] if src.suffix == ".cpp" else []
+    cmd = [HIPCC, *FLAGS, *lang, "-c", str(src), "-o", str(obj)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src.name}:\n{proc.stderr}")
+    return obj
+
+
+def build(verbose: bool = True) -> Path:
+    BUILD_DIR.mkdir(parents=True, exist_ok=True)
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        objs = list(pool.map(_compile, srcs))
+    cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(LIB_PATH)]
+    cmd += [str(o) for o in objs]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    if verbose:
+        print(f"built {LIB_PATH} from {len(srcs)} sources", file=sys.stderr)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,390 @@
+// Range-masked paged attention forward for gfx950.
+//
+// One workgroup (4 waves) owns 128 query rows of one (row, head); wave w owns
+// rows 32w..32w+31.  It walks the key tiles (64 keys) its rows can see and
+// keeps a running softmax per query row.  Everything is computed transposed:
+//
+//   S^T[kv, q] = K Q^T      A = K tile from LDS, B = Q held in registers
+//   O^T[d,  q] = V^T P^T    A = V^T tile from LDS, B = P^T straight from the
+//                           S^T accumulators
+//
+// With the 32x32x16 MFMA a lane holds one column of the accumulator, so in
+// this orientation a lane owns one query row: the row max / row sum need no
+// cross-lane reduction beyond one exchange between the two half-waves, the
+// rescale factor is a per-lane scalar, and the masked range of the row lives
+// in four registers.
+//
+// Key tiles are chosen per workgroup from the hull of its rows' ranges (tiles
+// no row can see are never loaded), each wave skips tiles outside its own
+// rows' hull, and a tile that lies inside every row's range of the wave skips
+// the per-element range test.
+#include <math.h>
+
+#include "attn_common.h"
+
+namespace dcp {
+
+struct AttnFwdParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  const int32_t* cu_seqlens_q;
+  const int32_t* cu_seqlens_kv;
+  const int32_t* attn_range;
+  const int32_t* q_block_table;
+  const int32_t* kv_block_table;
+  const int32_t* out_block_table;
+  const int32_t* row_order;
+  int n_ranges;
+  int batch;
+  int max_kv_blocks;
+  int total_q;
+  int block_size;
+  int n_heads_q;
+  int n_heads_kv;
+  int64_t kv_slot_stride;
+  int64_t kv_token_stride;
+  int n_out_slots;
+  int q_tiles_per_row;
+  float scale_log2;  // softmax_scale * log2(e)
+};
+
+constexpr int kFwdBM = 128;
+constexpr int kFwdBN = 64;
+constexpr int kFwdThreads = 256;
+
+template <int DTYPE, int D>
+__global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdParams p) {
+  constexpr int BN = kFwdBN;
+  constexpr int KS = D / 16;         // k-steps of S^T = K Q^T
+  constexpr int DT = D / 32;         // 32-row tiles of O^T
+  constexpr int K_STRIDE = D + 8;    // elements; 16-byte reads of 16 lanes hit 64 distinct banks
+  constexpr int VT_STRIDE = BN + 8;  // elements
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[BN * K_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[D * VT_STRIDE];
+  __shared__ int hull_lds[4][4];
+
+  const int tid = threadIdx.x;
+  const int w = tid >> 6;
+  const int lane = tid & 63;
+  const int c = lane & 31;
+  const int h = lane >> 5;
+
+  // ---- which (row, head, q tile) ----------------------------------------
+  int wg = blockIdx.x;
+  const int qt = wg % p.q_tiles_per_row;
+  wg /= p.q_tiles_per_row;
+  const int head = wg % p.n_heads_q;
+  const int bi = wg / p.n_heads_q;
+  const int b = p.row_order ? p.row_order[bi] : bi;
+  const int q_begin = p.cu_seqlens_q[b];
+  const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
+  const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
+  if (qt * kFwdBM >= seqlen_q) return;
+  const int kv_head = head / (p.n_heads_q / p.n_heads_kv);
+  const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
+
+  const int q_local = qt * kFwdBM + w * 32 + c;
+  const bool q_valid = q_local < seqlen_q;
+
+  // ---- Q fragment (B operand of S^T) ---------------------------------------
+  u32x4 qreg[KS];
+  {
+    const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) +
+                         ((int64_t)p.q_block_table[b] * p.block_size + q_local) * q_row_stride +
+                         (int64_t)head * D + h * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 z = {0, 0, 0, 0};
+      qreg[ks] = q_valid ? *reinterpret_cast<const u32x4*>(qp + ks * 16) : z;
+    }
+  }
+
+  // ---- this lane's query row: ranges ---------------------------------------
+  RangePair rng = {0, 0, 0, 0};
+  if (q_valid) {
+    const int32_t* r = p.attn_range + q_begin + q_local;
+    const int s0 = r[0], e0 = min(r[p.total_q], seqlen_kv);
+    rng.s0 = s0;
+    rng.len0 = max(e0 - s0, 0);
+    if (p.n_ranges == 2) {
+      const int s1 = r[2 * (int64_t)p.total_q], e1 = min(r[3 * (int64_t)p.total_q], seqlen_kv);
+      rng.s1 = s1;
+      rng.len1 = max(e1 - s1, 0);
+    }
+  }
+  // hull (what any row of the wave can see) and core (what every row sees)
+  const int big = 0x7fffffff;
+  const int w_lo0 = wave_min(rng.len0 > 0 ? rng.s0 : big);
+  const int w_hi0 = wave_max(rng.len0 > 0 ? rng.s0 + rng.len0 : 0);
+  const int w_lo1 = wave_min(rng.len1 > 0 ? rng.s1 : big);
+  const int w_hi1 = wave_max(rng.len1 > 0 ? rng.s1 + rng.len1 : 0);
+  const int core_lo0 = wave_max(rng.len0 > 0 ? rng.s0 : big);
+  const int core_hi0 = wave_min(rng.len0 > 0 ? rng.s0 + rng.len0 : 0);
+  const int core_lo1 = wave_max(rng.len1 > 0 ? rng.s1 : big);
+  const int core_hi1 = wave_min(rng.len1 > 0 ? rng.s1 + rng.len1 : 0);
+  if (lane == 0) {
+    hull_lds[w][0] = w_lo0;
+    hull_lds[w][1] = w_hi0;
+    hull_lds[w][2] = w_lo1;
+    hull_lds[w][3] = w_hi1;
+  }
+  __syncthreads();
+  int g_lo0 = big, g_hi0 = 0, g_lo1 = big, g_hi1 = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    g_lo0 = min(g_lo0, hull_lds[i][0]);
+    g_hi0 = max(g_hi0, hull_lds[i][1]);
+    g_lo1 = min(g_lo1, hull_lds[i][2]);
+    g_hi1 = max(g_hi1, hull_lds[i][3]);
+  }
+  const int kt_begin = min(g_lo0, g_lo1) / BN;
+  const int kt_end = (max(g_hi0, g_hi1) + BN - 1) / BN;  // 0 when nothing is visible
+
+  // ---- running state ---------------------------------------------------------
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o_acc[dt][i] = 0.0f;
+  float m_run = -INFINITY;  // running max, log2 domain
+  float l_run = 0.0f;       // this half-wave's partial row sum
+
+  const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
+  const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
+  const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
+
+  // global -> LDS staging maps
+  constexpr int CH = D / 8;                    // 16-byte chunks per row
+  constexpr int K_ROWS_PER_PASS = kFwdThreads / CH;
+  constexpr int K_PASSES = BN / K_ROWS_PER_PASS;
+  constexpr int V_UNITS = (BN / 4) * CH;       // (4 keys) x (8 dims) units
+  constexpr int V_PASSES = (V_UNITS + kFwdThreads - 1) / kFwdThreads;
+  const int k_row = tid / CH, k_chunk = tid % CH;
+
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int k0 = kt * BN;
+    const bool wg_active = (k0 < g_hi0 && k0 + BN > g_lo0) || (k0 < g_hi1 && k0 + BN > g_lo1);
+    if (!wg_active) continue;
+
+    // ---- stage K (row-major) and V (transposed, k-slot order) into LDS ------
+    const int blk = k0 / p.block_size;
+    const int tok0 = k0 - blk * p.block_size;
+    const int64_t tile_off = (int64_t)kv_table[blk] * p.kv_slot_stride + (int64_t)tok0 * p.kv_token_stride;
+    u32x4 kst[K_PASSES];
+#pragma unroll
+    for (int ps = 0; ps < K_PASSES; ++ps) {
+      const int r = ps * K_ROWS_PER_PASS + k_row;
+      kst[ps] = *reinterpret_cast<const u32x4*>(kg + tile_off + (int64_t)r * p.kv_token_stride + k_chunk * 8);
+    }
+    u32x4 vst[V_PASSES][4];
+#pragma unroll
+    for (int ps = 0; ps < V_PASSES; ++ps) {
+      const int u = ps * kFwdThreads + tid;
+      if (u < V_UNITS) {
+        const int kvg = u % (BN / 4), dg = u / (BN / 4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          vst[ps][r] = *reinterpret_cast<const u32x4*>(
+              vg + tile_off + (int64_t)(kvg * 4 + r) * p.kv_token_stride + dg * 8);
+      }
+    }
+    __syncthreads();  // everyone is done reading the previous tile
+#pragma unroll
+    for (int ps = 0; ps < K_PASSES; ++ps) {
+      const int r = ps * K_ROWS_PER_PASS + k_row;
+      *reinterpret_cast<u32x4*>(&k_lds[r * K_STRIDE + k_chunk * 8]) = kst[ps];
+    }
+#pragma unroll
+    for (int ps = 0; ps < V_PASSES; ++ps) {
+      const int u = ps * kFwdThreads + tid;
+      if (u < V_UNITS) {
+        const int kvg = u % (BN / 4), dg = u / (BN / 4);
+        const int pos = (kvg / 4) * 16 + kslot_pos(kvg % 4);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t a0 = vst[ps][0][m], a1 = vst[ps][1][m], a2 = vst[ps][2][m], a3 = vst[ps][3][m];
+          u32x2 even = {(a0 & 0xffffu) | (a1 << 16), (a2 & 0xffffu) | (a3 << 16)};
+          u32x2 odd = {(a0 >> 16) | (a1 & 0xffff0000u), (a2 >> 16) | (a3 & 0xffff0000u)};
+          *reinterpret_cast<u32x2*>(&vt_lds[(dg * 8 + 2 * m) * VT_STRIDE + pos]) = even;
+          *reinterpret_cast<u32x2*>(&vt_lds[(dg * 8 + 2 * m + 1) * VT_STRIDE + pos]) = odd;
+        }
+      }
+    }
+    __syncthreads();
+
+    const bool wave_active = (k0 < w_hi0 && k0 + BN > w_lo0) || (k0 < w_hi1 && k0 + BN > w_lo1);
+    if (!wave_active) continue;
+
+    // ---- S^T = K Q^T ----------------------------------------------------------
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_acc[nt][i] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(&k_lds[(nt * 32 + c) * K_STRIDE + ks * 16 + h * 8]);
+        s_acc[nt] = mfma_32x32x16<DTYPE>(a, qreg[ks], s_acc[nt]);
+      }
+    }
+
+    // ---- online softmax (log2 domain) -----------------------------------------
+    const bool unmasked = (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
+    float mx = -INFINITY;
+    if (unmasked) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[nt][i]);
+      mx *= p.scale_log2;
+    } else {
+      const int kb = k0 + 4 * h;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int kv = kb + nt * 32 + 8 * (i / 4) + (i % 4);
+          const float s = rng.contains(kv) ? s_acc[nt][i] : -INFINITY;
+          s_acc[nt][i] = s;
+          mx = fmaxf(mx, s);
+        }
+      mx *= p.scale_log2;  // -inf stays -inf (scale > 0)
+    }
+    mx = fmaxf(mx, xor32(mx));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+    if (__any(m_new > m_run)) {
+      const float alpha = exp2f(m_run - m_use);  // m_run = -inf -> 0
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[dt][i] *= alpha;
+    }
+    m_run = m_new;
+
+    u32x4 pb[4];
+    float lsum = 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        float e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          e[j] = exp2f(fmaf(s_acc[nt][g * 8 + j], p.scale_log2, -m_use));
+          lsum += e[j];
+        }
+        u32x4 packed = {pack2<DTYPE>(e[0], e[1]), pack2<DTYPE>(e[2], e[3]), pack2<DTYPE>(e[4], e[5]),
+                        pack2<DTYPE>(e[6], e[7])};
+        pb[nt * 2 + g] = packed;
+      }
+    l_run += lsum;
+
+    // ---- O^T += V^T P^T ---------------------------------------------------------
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int s2 = 0; s2 < 4; ++s2) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(&vt_lds[(dt * 32 + c) * VT_STRIDE + s2 * 16 + h * 8]);
+        o_acc[dt] = mfma_32x32x16<DTYPE>(a, pb[s2], o_acc[dt]);
+      }
+  }
+
+  // ---- epilogue ------------------------------------------------------------------
+  const float l_tot = l_run + xor32(l_run);
+  if (!q_valid) return;
+  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+  const int o_slot = p.out_block_table[b];
+  uint16_t* op = reinterpret_cast<uint16_t*>(p.out) +
+                 ((int64_t)o_slot * p.block_size + q_local) * q_row_stride + (int64_t)head * D + 4 * h;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 pk = {pack2<DTYPE>(o_acc[dt][4 * g] * inv, o_acc[dt][4 * g + 1] * inv),
+                  pack2<DTYPE>(o_acc[dt][4 * g + 2] * inv, o_acc[dt][4 * g + 3] * inv)};
+      *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * g) = pk;
+    }
+  if (h == 0) {
+    const float lse = l_tot > 0.0f ? (m_run + log2f(l_tot)) * kLn2 : INFINITY;
+    p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local] = lse;
+  }
+}
+
+}  // namespace dcp
+
+using namespace dcp;
+
+extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                            const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_kv,
+                            const int32_t* attn_range, int n_ranges, const int32_t* q_block_table,
+                            const int32_t* kv_block_table, const int32_t* out_block_table,
+                            const int32_t* row_order, int batch, int max_kv_blocks, int total_q,
+                            int block_size, int n_heads_q, int n_heads_kv, int head_dim,
+                            int64_t kv_slot_stride, int64_t kv_token_stride, int n_out_slots,
+                            float softmax_scale, int dtype, void* stream) {
+  if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
+    return fail(DCP_ERR_UNSUPPORTED, "attn_fwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
+  if (head_dim != 64 && head_dim != 128)
+    return fail(DCP_ERR_UNSUPPORTED, "attn_fwd: head_dim %d unsupported (64 or 128)", head_dim);
+  DCP_REQUIRE(n_ranges == 1 || n_ranges == 2, "attn_fwd: n_ranges must be 1 or 2, got %d", n_ranges);
+  DCP_REQUIRE(batch >= 0 && total_q >= 0, "attn_fwd: negative size");
+  DCP_REQUIRE(softmax_scale > 0.0f, "attn_fwd: softmax_scale must be positive");
+  if (batch == 0) return DCP_OK;
+  DCP_REQUIRE(block_size > 0 && block_size % kFwdBN == 0,
+              "attn_fwd: block_size %d must be a positive multiple of %d", block_size, kFwdBN);
+  DCP_REQUIRE(n_heads_q > 0 && n_heads_kv > 0 && n_heads_q % n_heads_kv == 0,
+              "attn_fwd: n_heads_q %d must be a multiple of n_heads_kv %d", n_heads_q, n_heads_kv);
+  DCP_REQUIRE(max_kv_blocks > 0 && n_out_slots > 0, "attn_fwd: empty block tables");
+  DCP_REQUIRE(kv_token_stride % 8 == 0 && kv_slot_stride % 8 == 0,
+              "attn_fwd: kv strides must be multiples of 8 elements");
+  DCP_REQUIRE(q && k && v && out && lse && cu_seqlens_q && cu_seqlens_kv && attn_range &&
+                  q_block_table && kv_block_table && out_block_table,
+              "attn_fwd: null argument");
+  DCP_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+                reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) & 15) == 0,
+              "attn_fwd: q/k/v/out must be 16-byte aligned");
+  AttnFwdParams p;
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.out = out;
+  p.lse = lse;
+  p.cu_seqlens_q = cu_seqlens_q;
+  p.cu_seqlens_kv = cu_seqlens_kv;
+  p.attn_range = attn_range;
+  p.q_block_table = q_block_table;
+  p.kv_block_table = kv_block_table;
+  p.out_block_table = out_block_table;
+  p.row_order = row_order;
+  p.n_ranges = n_ranges;
+  p.batch = batch;
+  p.max_kv_blocks = max_kv_blocks;
+  p.total_q = total_q;
+  p.block_size = block_size;
+  p.n_heads_q = n_heads_q;
+  p.n_heads_kv = n_heads_kv;
+  p.kv_slot_stride = kv_slot_stride;
+  p.kv_token_stride = kv_token_stride;
+  p.n_out_slots = n_out_slots;
+  p.q_tiles_per_row = (block_size + kFwdBM - 1) / kFwdBM;
+  p.scale_log2 = softmax_scale * kLog2e;
+  const int64_t n_wg = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
+  DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_fwd: grid too large");
+  dim3 grid((unsigned)n_wg), block(kFwdThreads);
+#define DCP_FWD(DT, HD) \
+  hipLaunchKernelGGL((attn_fwd_kernel<DT, HD>), grid, block, 0, (hipStream_t)stream, p)
+  if (dtype == DCP_DTYPE_BF16) {
+    if (head_dim == 128) DCP_FWD(DCP_DTYPE_BF16, 128);
+    else DCP_FWD(DCP_DTYPE_BF16, 64);
+  } else {
+    if (head_dim == 128) DCP_FWD(DCP_DTYPE_FP16, 128);
+    else DCP_FWD(DCP_DTYPE_FP16, 64);
+  }
+#undef DCP_FWD
+  return check_launch("attn_fwd_kernel");
+}

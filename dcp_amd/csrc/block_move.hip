@@ -1,0 +1,169 @@
+// Block gather/scatter kernels: pointer-table block copy, per-token dKV copy
+// and head-strided LSE copy.  Pure byte movement, HBM-bound.
+//
+// One workgroup of 256 lanes moves one 16 KiB chunk of one block: every lane
+// issues four independent 16-byte loads before its four stores, so a wave has
+// 4 KiB in flight and consecutive lanes touch consecutive 16-byte words.
+#include "common.h"
+
+namespace dcp {
+
+constexpr int kCopyThreads = 256;
+constexpr int kCopyUnroll = 4;
+constexpr int kCopyChunkBytes = kCopyThreads * 16 * kCopyUnroll;  // 16 KiB
+
+// Tables are nullable where the dKV variant has no such column: a null
+// offset/stride table means offset 0, and n_count[p] is multiplied by
+// `elems_per_count` (1 for the element-count variant, per_token_size for the
+// token-count variant).
+__global__ __launch_bounds__(kCopyThreads) void copy_varlen_kernel(
+    const int64_t* __restrict__ src_ptrs, const int32_t* __restrict__ src_offsets,
+    const int32_t* __restrict__ src_strides, const int64_t* __restrict__ dst_ptrs,
+    const int32_t* __restrict__ dst_offsets, const int32_t* __restrict__ dst_strides,
+    const int32_t* __restrict__ n_count, int64_t elems_per_count,
+    int chunks_per_block, int elem_size) {
+  const int p = blockIdx.x / chunks_per_block;
+  const int c = blockIdx.x - p * chunks_per_block;
+  const int64_t n_bytes = (int64_t)n_count[p] * elems_per_count * elem_size;
+  const int64_t begin = (int64_t)c * kCopyChunkBytes;
+  if (begin >= n_bytes) return;
+  const int64_t end = min(begin + (int64_t)kCopyChunkBytes, n_bytes);
+
+  int64_t src_off = 0, dst_off = 0;
+  if (src_offsets) src_off = (int64_t)src_offsets[p] * src_strides[p] * elem_size;
+  if (dst_offsets) dst_off = (int64_t)dst_offsets[p] * dst_strides[p] * elem_size;
+  const char* src = reinterpret_cast<const char*>(src_ptrs[p]) + src_off;
+  char* dst = reinterpret_cast<char*>(dst_ptrs[p]) + dst_off;
+
+  const bool aligned =
+      ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+  if (aligned) {
+    const int64_t vec_end = begin + ((end - begin) & ~(int64_t)15);
+    const u32x4* s = reinterpret_cast<const u32x4*>(src + begin);
+    u32x4* d = reinterpret_cast<u32x4*>(dst + begin);
+    const int n_vec = (int)((vec_end - begin) >> 4);
+    if (n_vec == kCopyThreads * kCopyUnroll) {
+      u32x4 r[kCopyUnroll];
+#pragma unroll
+      for (int u = 0; u < kCopyUnroll; ++u)
+        r[u] = __builtin_nontemporal_load(s + threadIdx.x + u * kCopyThreads);
+#pragma unroll
+      for (int u = 0; u < kCopyUnroll; ++u)
+        __builtin_nontemporal_store(r[u], d + threadIdx.x + u * kCopyThreads);
+    } else {
+      for (int i = threadIdx.x; i < n_vec; i += kCopyThreads) d[i] = s[i];
+    }
+    // sub-16-byte tail of the block (only in its last chunk)
+    for (int64_t b = vec_end + threadIdx.x * elem_size; b < end;
+         b += (int64_t)kCopyThreads * elem_size) {
+      if (elem_size == 2)
+        *reinterpret_cast<uint16_t*>(dst + b) = *reinterpret_cast<const uint16_t*>(src + b);
+      else
+        *reinterpret_cast<uint32_t*>(dst + b) = *reinterpret_cast<const uint32_t*>(src + b);
+    }
+  } else {
+    for (int64_t b = begin + (int64_t)threadIdx.x * elem_size; b < end;
+         b += (int64_t)kCopyThreads * elem_size) {
+      if (elem_size == 2)
+        *reinterpret_cast<uint16_t*>(dst + b) = *reinterpret_cast<const uint16_t*>(src + b);
+      else
+        *reinterpret_cast<uint32_t*>(dst + b) = *reinterpret_cast<const uint32_t*>(src + b);
+    }
+  }
+}
+
+// grid: (blocks, heads, token chunks); LSE rows are short and arbitrarily
+// aligned, so this is a plain coalesced element copy.
+template <typename T>
+__global__ __launch_bounds__(256) void copy_lse_kernel(
+    const int64_t* __restrict__ src_ptrs, const int32_t* __restrict__ src_token_offsets,
+    const int32_t* __restrict__ src_head_strides, const int64_t* __restrict__ dst_ptrs,
+    const int32_t* __restrict__ dst_token_offsets,
+    const int32_t* __restrict__ dst_head_strides, const int32_t* __restrict__ n_tokens) {
+  const int p = blockIdx.x;
+  const int h = blockIdx.y;
+  const int t = blockIdx.z * 256 + threadIdx.x;
+  if (t >= n_tokens[p]) return;
+  const T* src = reinterpret_cast<const T*>(src_ptrs[p]) +
+                 (int64_t)h * src_head_strides[p] + src_token_offsets[p];
+  T* dst = reinterpret_cast<T*>(dst_ptrs[p]) + (int64_t)h * dst_head_strides[p] +
+           dst_token_offsets[p];
+  dst[t] = src[t];
+}
+
+static int launch_copy(const int64_t* src_ptrs, const int32_t* src_offsets,
+                       const int32_t* src_strides, const int64_t* dst_ptrs,
+                       const int32_t* dst_offsets, const int32_t* dst_strides,
+                       const int32_t* n_count, int64_t elems_per_count, int n_ptrs,
+                       int64_t block_numel, int elem_size, void* stream) {
+  const int64_t block_bytes = block_numel * elem_size;
+  const int64_t chunks = (block_bytes + kCopyChunkBytes - 1) / kCopyChunkBytes;
+  DCP_REQUIRE(chunks * n_ptrs < (int64_t)1 << 31, "copy grid too large: %lld blocks x %lld chunks",
+              (long long)n_ptrs, (long long)chunks);
+  hipLaunchKernelGGL(copy_varlen_kernel, dim3((unsigned)(chunks * n_ptrs)), dim3(kCopyThreads), 0,
+                     (hipStream_t)stream, src_ptrs, src_offsets, src_strides, dst_ptrs,
+                     dst_offsets, dst_strides, n_count, elems_per_count, (int)chunks, elem_size);
+  return check_launch("copy_varlen_kernel");
+}
+
+}  // namespace dcp
+
+using namespace dcp;
+
+extern "C" int dcp_fused_copy_varlen(const int64_t* src_ptrs, const int32_t* src_offsets,
+                                     const int32_t* src_strides, const int64_t* dst_ptrs,
+                                     const int32_t* dst_offsets, const int32_t* dst_strides,
+                                     const int32_t* n_elements, int n_ptrs, int64_t block_numel,
+                                     int elem_size, void* stream) {
+  DCP_REQUIRE(elem_size == 2 || elem_size == 4, "copy: unsupported element size %d", elem_size);
+  DCP_REQUIRE(n_ptrs >= 0 && block_numel >= 0, "copy: negative size");
+  if (n_ptrs == 0 || block_numel == 0) return DCP_OK;
+  DCP_REQUIRE(src_ptrs && dst_ptrs && src_offsets && src_strides && dst_offsets && dst_strides &&
+                  n_elements,
+              "copy: null table");
+  return launch_copy(src_ptrs, src_offsets, src_strides, dst_ptrs, dst_offsets, dst_strides,
+                     n_elements, 1, n_ptrs, block_numel, elem_size, stream);
+}
+
+extern "C" int dcp_fused_copy_varlen_dkv(const int64_t* src_ptrs, const int64_t* dst_ptrs,
+                                         const int32_t* n_tokens, int n_ptrs, int max_n_tokens,
+                                         int per_token_size, int elem_size, void* stream) {
+  DCP_REQUIRE(elem_size == 2 || elem_size == 4, "dkv copy: unsupported element size %d",
+              elem_size);
+  DCP_REQUIRE(n_ptrs >= 0 && max_n_tokens >= 0 && per_token_size >= 0, "dkv copy: negative size");
+  if (n_ptrs == 0 || max_n_tokens == 0 || per_token_size == 0) return DCP_OK;
+  DCP_REQUIRE(src_ptrs && dst_ptrs && n_tokens, "dkv copy: null table");
+  return launch_copy(src_ptrs, nullptr, nullptr, dst_ptrs, nullptr, nullptr, n_tokens,
+                     per_token_size, n_ptrs, (int64_t)max_n_tokens * per_token_size, elem_size,
+                     stream);
+}
+
+extern "C" int dcp_fused_copy_varlen_lse(const int64_t* src_ptrs,
+                                         const int32_t* src_token_offsets,
+                                         const int32_t* src_head_strides, const int64_t* dst_ptrs,
+                                         const int32_t* dst_token_offsets,
+                                         const int32_t* dst_head_strides, const int32_t* n_tokens,
+                                         int n_ptrs, int head_block_size, int max_n_tokens,
+                                         int elem_size, void* stream) {
+  DCP_REQUIRE(elem_size == 2 || elem_size == 4, "lse copy: unsupported element size %d",
+              elem_size);
+  DCP_REQUIRE(n_ptrs >= 0 && head_block_size >= 0 && max_n_tokens >= 0,
+              "lse copy: negative size");
+  if (n_ptrs == 0 || head_block_size == 0 || max_n_tokens == 0) return DCP_OK;
+  DCP_REQUIRE(head_block_size <= 65535 && max_n_tokens <= 65535 * 256,
+              "lse copy: head_block_size %d or max_n_tokens %d too large", head_block_size,
+              max_n_tokens);
+  DCP_REQUIRE(src_ptrs && dst_ptrs && src_token_offsets && src_head_strides &&
+                  dst_token_offsets && dst_head_strides && n_tokens,
+              "lse copy: null table");
+  dim3 grid(n_ptrs, head_block_size, (max_n_tokens + 255) / 256);
+  if (elem_size == 4)
+    hipLaunchKernelGGL(copy_lse_kernel<uint32_t>, grid, dim3(256), 0, (hipStream_t)stream,
+                       src_ptrs, src_token_offsets, src_head_strides, dst_ptrs, dst_token_offsets,
+                       dst_head_strides, n_tokens);
+  else
+    hipLaunchKernelGGL(copy_lse_kernel<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream,
+                       src_ptrs, src_token_offsets, src_head_strides, dst_ptrs, dst_token_offsets,
+                       dst_head_strides, n_tokens);
+  return check_launch("copy_lse_kernel");
+}

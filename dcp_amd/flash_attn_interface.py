@@ -1,0 +1,242 @@
+"""Range-masked paged variable-length attention: the two functions the
+reference executor imports from its flash-attention fork
+(``dcp_flash_attn.flash_attn_interface._flash_attn_varlen_forward`` /
+``_flash_attn_varlen_backward``, called at
+``dcp/runtime/flash_attention/executor.py:161-184`` and ``:303-334``), with the
+same argument order, backed by the gfx950 kernels of ``libdcp_hip.so``.
+
+Only the configuration the executor uses is implemented: no dropout, no causal
+flag, no sliding window, no softcap, no alibi; masking comes from
+``attn_range`` and all tensors are paged through block tables.  Anything else
+raises ``NotImplementedError`` rather than computing something different.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from dcp_amd import _lib
+from dcp_amd.ops.fused_ops import dtype_code
+
+__all__ = ["_flash_attn_varlen_forward", "_flash_attn_varlen_backward"]
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap,
+                 alibi_slopes, return_softmax=False):
+    if dropout_p != 0.0:
+        raise NotImplementedError("dropout is not supported")
+    if causal:
+        raise NotImplementedError("use attn_range instead of the causal flag")
+    if window_size_left != -1 or window_size_right != -1:
+        raise NotImplementedError("use attn_range instead of window_size")
+    if softcap != 0.0:
+        raise NotImplementedError("softcap is not supported")
+    if alibi_slopes is not None:
+        raise NotImplementedError("alibi is not supported")
+    if return_softmax:
+        raise NotImplementedError("return_softmax is not supported")
+
+
+def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous int32 device tensor")
+    return t
+
+
+def _kv_strides(k: torch.Tensor, v: torch.Tensor, name: str):
+    """k and v are [n_slots, block_size, n_heads_kv, D] views (typically the
+    two halves of a [n_slots, block_size, 2, n_heads_kv, D] buffer)."""
+    if k.shape != v.shape or k.stride() != v.stride():
+        raise ValueError(f"{name}: k and v must have the same shape and strides")
+    if k.dim() != 4:
+        raise ValueError(f"{name}: k/v must be paged [n_slots, block_size, n_heads_kv, D]")
+    if k.stride(3) != 1 or k.stride(2) != k.shape[3]:
+        raise ValueError(f"{name}: k/v head and feature axes must be dense")
+    return k.stride(0), k.stride(1)
+
+
+def _range_arg(attn_range: torch.Tensor, total_q: int):
+    _i32(attn_range, "attn_range")
+    if attn_range.dim() == 2 and tuple(attn_range.shape) == (2, total_q):
+        return 1
+    if attn_range.dim() == 3 and tuple(attn_range.shape) == (2, 2, total_q):
+        return 2
+    raise ValueError(
+        f"attn_range must be [2, {total_q}] or [2, 2, {total_q}], got {tuple(attn_range.shape)}"
+    )
+
+
+def _flash_attn_varlen_forward(
+    q,
+    k,
+    v,
+    cu_seqlens_q,
+    cu_seqlens_k,
+    total_q,
+    max_seqlen_q,
+    max_seqlen_k,
+    dropout_p,
+    softmax_scale,
+    causal=False,
+    window_size_left=-1,
+    window_size_right=-1,
+    softcap=0.0,
+    alibi_slopes=None,
+    return_softmax=False,
+    attn_range=None,
+    q_block_table=None,
+    kv_block_table=None,
+    out_block_table=None,
+    out_=None,
+    lse_=None,
+    row_order: Optional[torch.Tensor] = None,
+):
+    """Writes the row outputs into ``out_`` / ``lse_`` in place and returns
+    ``(out_, lse_, None, None)`` (the reference returns
+    ``out_padded, softmax_lse, S_dmask, rng_state``).
+
+    q ``[n_slots, bs, H, D]``; k, v ``[n_slots, bs, Hkv, D]`` views; block
+    tables int32 ``[B, 1]`` (q, out) and ``[B, max_blocks]`` (kv, padded with
+    -1); ``attn_range`` int32 ``[2, total_q]`` or ``[2, 2, total_q]``;
+    ``out_`` like q; ``lse_`` fp32 ``[H, n_out_slots, bs]``.
+    ``row_order`` (extension): launch order of the rows, longest first.
+    """
+    _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap,
+                 alibi_slopes, return_softmax)
+    if attn_range is None or q_block_table is None or kv_block_table is None \
+            or out_block_table is None or out_ is None or lse_ is None:
+        raise NotImplementedError(
+            "only the paged, range-masked, in-place form is implemented")
+    if q.dim() != 4 or not q.is_contiguous() or not out_.is_contiguous():
+        raise ValueError("q and out_ must be contiguous [n_slots, block_size, H, D]")
+    if lse_.dtype != torch.float32 or not lse_.is_contiguous():
+        raise ValueError("lse_ must be contiguous float32 [H, n_out_slots, block_size]")
+    _, block_size, n_heads_q, head_dim = q.shape
+    n_heads_kv = k.shape[2]
+    kv_slot_stride, kv_token_stride = _kv_strides(k, v, "forward")
+    n_ranges = _range_arg(attn_range, total_q)
+    batch = cu_seqlens_q.numel() - 1
+    if tuple(lse_.shape) != (n_heads_q, out_.shape[0], block_size):
+        raise ValueError(f"lse_ shape {tuple(lse_.shape)} does not match out_")
+    if softmax_scale is None:
+        softmax_scale = head_dim ** (-0.5)
+    _lib.call(
+        "dcp_attn_fwd",
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out_.data_ptr(), lse_.data_ptr(),
+        _i32(cu_seqlens_q, "cu_seqlens_q").data_ptr(),
+        _i32(cu_seqlens_k, "cu_seqlens_k").data_ptr(),
+        attn_range.data_ptr(), n_ranges,
+        _i32(q_block_table, "q_block_table").data_ptr(),
+        _i32(kv_block_table, "kv_block_table").data_ptr(),
+        _i32(out_block_table, "out_block_table").data_ptr(),
+        0 if row_order is None else _i32(row_order, "row_order").data_ptr(),
+        batch, kv_block_table.shape[1], int(total_q), block_size,
+        n_heads_q, n_heads_kv, head_dim,
+        kv_slot_stride, kv_token_stride, out_.shape[0],
+        float(softmax_scale), dtype_code(q.dtype), _stream(),
+    )
+    return out_, lse_, None, None
+
+
+def _flash_attn_varlen_backward(
+    dout,
+    q,
+    k,
+    v,
+    out,
+    softmax_lse,
+    dq,
+    dk,
+    dv,
+    cu_seqlens_q,
+    cu_seqlens_k,
+    total_q,
+    total_k,
+    max_seqlen_q,
+    max_seqlen_k,
+    dropout_p,
+    softmax_scale,
+    causal,
+    window_size_left,
+    window_size_right,
+    softcap,
+    alibi_slopes,
+    deterministic,
+    attn_range=None,
+    q_block_table=None,
+    kv_block_table=None,
+    out_block_table=None,
+    dq_block_table=None,
+    dkv_block_table=None,
+    rng_state=None,
+    dq_accum: Optional[torch.Tensor] = None,
+    delta: Optional[torch.Tensor] = None,
+    row_order: Optional[torch.Tensor] = None,
+):
+    """Writes dQ into ``dq`` (slots ``dq_block_table``) and dK/dV into
+    ``dk``/``dv`` (one slot per (row, kv block), ``dkv_block_table``).
+    dK/dV of a kv head are summed over the q heads of its group inside the
+    kernel, and every token of a dK/dV slot is written, so ``dk``/``dv`` need
+    not be zeroed.
+
+    ``dq_accum`` (fp32, ``total_q * H * D`` elements) and ``delta`` (fp32,
+    ``total_q * H``) are scratch; pass preallocated tensors to keep the call
+    allocation-free (e.g. under graph capture), otherwise they are allocated
+    here.
+    """
+    _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap, alibi_slopes)
+    if attn_range is None or q_block_table is None or kv_block_table is None \
+            or out_block_table is None or dq_block_table is None or dkv_block_table is None:
+        raise NotImplementedError(
+            "only the paged, range-masked form is implemented")
+    for name, t in (("q", q), ("out", out), ("dout", dout), ("dq", dq)):
+        if t.dim() != 4 or not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous [n_slots, block_size, H, D]")
+    _, block_size, n_heads_q, head_dim = q.shape
+    n_heads_kv = k.shape[2]
+    kv_slot_stride, kv_token_stride = _kv_strides(k, v, "backward k/v")
+    dkv_slot_stride, dkv_token_stride = _kv_strides(dk, dv, "backward dk/dv")
+    n_ranges = _range_arg(attn_range, total_q)
+    batch = cu_seqlens_q.numel() - 1
+    if softmax_lse.dtype != torch.float32 or not softmax_lse.is_contiguous():
+        raise ValueError("softmax_lse must be contiguous float32")
+    if tuple(softmax_lse.shape) != (n_heads_q, out.shape[0], block_size):
+        raise ValueError(f"softmax_lse shape {tuple(softmax_lse.shape)} does not match out")
+    if dout.shape[0] != out.shape[0]:
+        raise ValueError("dout and out must have the same number of slots")
+    if softmax_scale is None:
+        softmax_scale = head_dim ** (-0.5)
+    n_acc = int(total_q) * n_heads_q * head_dim
+    if dq_accum is None:
+        dq_accum = torch.empty(n_acc, dtype=torch.float32, device=q.device)
+    if delta is None:
+        delta = torch.empty(int(total_q) * n_heads_q, dtype=torch.float32, device=q.device)
+    if dq_accum.dtype != torch.float32 or dq_accum.numel() < n_acc:
+        raise ValueError("dq_accum must be float32 with total_q*H*D elements")
+    if delta.dtype != torch.float32 or delta.numel() < int(total_q) * n_heads_q:
+        raise ValueError("delta must be float32 with total_q*H elements")
+    _lib.call(
+        "dcp_attn_bwd",
+        dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+        softmax_lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+        dq_accum.data_ptr(), delta.data_ptr(),
+        _i32(cu_seqlens_q, "cu_seqlens_q").data_ptr(),
+        _i32(cu_seqlens_k, "cu_seqlens_k").data_ptr(),
+        attn_range.data_ptr(), n_ranges,
+        _i32(q_block_table, "q_block_table").data_ptr(),
+        _i32(kv_block_table, "kv_block_table").data_ptr(),
+        _i32(out_block_table, "out_block_table").data_ptr(),
+        _i32(dq_block_table, "dq_block_table").data_ptr(),
+        _i32(dkv_block_table, "dkv_block_table").data_ptr(),
+        batch, kv_block_table.shape[1], int(total_q), block_size,
+        n_heads_q, n_heads_kv, head_dim,
+        kv_slot_stride, kv_token_stride, dkv_slot_stride, dkv_token_stride,
+        out.shape[0], float(softmax_scale), dtype_code(q.dtype), _stream(),
+    )
+    return dq, dk, dv, None

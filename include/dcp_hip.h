@@ -1,0 +1,214 @@
+/*
+ * C ABI of libdcp_hip.so: the gfx950 kernels behind DCP's per-device blockwise
+ * attention executor.
+ *
+ * Conventions
+ *  - every pointer marked "device" is a HIP device address on the current
+ *    device; "host" pointers are ordinary host memory read before return;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream); all
+ *    work is enqueued on it and nothing synchronises with the host;
+ *  - the library borrows memory for the duration of a launch: it allocates
+ *    nothing and keeps no pointer;
+ *  - return value 0 = launched, nonzero = rejected before any launch (argument
+ *    error); dcp_last_error() then returns a message for the calling thread;
+ *  - dtype codes follow the reference's wire integers
+ *    (dcp/core/serialization.py:410-437): 0 bf16, 1 fp16, 2 fp32.
+ *
+ * Each entry point names the reference interface it replaces.
+ */
+#ifndef DCP_HIP_H_
+#define DCP_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DCP_DTYPE_BF16 0
+#define DCP_DTYPE_FP16 1
+#define DCP_DTYPE_FP32 2
+
+#define DCP_OK 0
+#define DCP_ERR_ARG 1
+#define DCP_ERR_UNSUPPORTED 2
+#define DCP_ERR_LAUNCH 3
+
+/* Library / ABI version (major*100 + minor). */
+int dcp_version(void);
+
+/* Message of the last nonzero return on this thread ("" if none). */
+const char* dcp_last_error(void);
+
+/*
+ * Block gather / scatter through pointer tables.
+ * Replaces dcp.ops.fused_ops.fused_copy_{bf16,fp16,fp32}_varlen
+ * (dcp/ops/fused_ops.py:842-864, 916-938, 1013-1035; kernels :290-335,
+ * :472-517, :654-699), called from _handle_memcpy
+ * (dcp/runtime/flash_attention/executor.py:793-805).
+ *
+ * For p in [0, n_ptrs), i in [0, n_elements[p]):
+ *   ((T*)dst_ptrs[p])[dst_offsets[p]*dst_strides[p] + i] =
+ *   ((T*)src_ptrs[p])[src_offsets[p]*src_strides[p] + i]
+ * T has `elem_size` bytes (2 or 4); offsets/strides are in elements.
+ * All seven tables are device int64/int32 arrays of length n_ptrs.
+ * `block_numel` is the padded block size in elements (upper bound of
+ * n_elements[p]); it only sizes the grid.
+ */
+int dcp_fused_copy_varlen(const int64_t* src_ptrs, const int32_t* src_offsets,
+                          const int32_t* src_strides, const int64_t* dst_ptrs,
+                          const int32_t* dst_offsets,
+                          const int32_t* dst_strides,
+                          const int32_t* n_elements, int n_ptrs,
+                          int64_t block_numel, int elem_size, void* stream);
+
+/*
+ * Copy the first n_tokens[p] tokens (per_token_size elements each) of block p.
+ * Replaces fused_copy_{bf16,fp16,fp32}_varlen_dkv (fused_ops.py:867-885,
+ * 941-959, 1038-1056; kernel :338-367), used after the GQA backward
+ * (executor.py:1102-1114).  src_ptrs/dst_ptrs address the blocks themselves.
+ */
+int dcp_fused_copy_varlen_dkv(const int64_t* src_ptrs, const int64_t* dst_ptrs,
+                              const int32_t* n_tokens, int n_ptrs,
+                              int max_n_tokens, int per_token_size,
+                              int elem_size, void* stream);
+
+/*
+ * Head-strided copy of log-sum-exp blocks.
+ * Replaces fused_copy_{bf16,fp16,fp32}_varlen_lse (fused_ops.py:888-913,
+ * 962-987, 1059-1084; kernel :370-429), called from _handle_memcpy
+ * (executor.py:806-810).
+ * For h < head_block_size, t < n_tokens[p]:
+ *   dst[p][h*dst_head_strides[p] + dst_token_offsets[p] + t] =
+ *   src[p][h*src_head_strides[p] + src_token_offsets[p] + t]
+ * Unlike the reference kernel, head_block_size need not be a power of two.
+ */
+int dcp_fused_copy_varlen_lse(const int64_t* src_ptrs,
+                              const int32_t* src_token_offsets,
+                              const int32_t* src_head_strides,
+                              const int64_t* dst_ptrs,
+                              const int32_t* dst_token_offsets,
+                              const int32_t* dst_head_strides,
+                              const int32_t* n_tokens, int n_ptrs,
+                              int head_block_size, int max_n_tokens,
+                              int elem_size, void* stream);
+
+/*
+ * N-way online-softmax merge of partial (out, lse) blocks, fused with the
+ * scatter into the destination.
+ * Replaces flash_attn_update_out_lse (fused_ops.py:149-247, kernel :15-146),
+ * called from _handle_reduction (executor.py:1299-1329).
+ *
+ * For op o, head h < n_head, token t < n_tokens_per_block[o], over the
+ * sources j < block_lengths[o] with block b_j = src_block_table[o*max_n+j]:
+ *   l_j   = src_lse[h*src_lse_head_stride + b_j*lse_block_stride + t*lse_token_stride]
+ *   sources with l_j = +-inf are ignored;
+ *   lse*  = m + log(sum_j exp(l_j - m)),  m = max_j l_j
+ *   out*  = sum_j exp(l_j - lse*) * src_out[b_j*out_block_stride + t*out_token_stride + h*head_dim + :]
+ *   no finite source: lse* = -1, out* = 0.
+ * dst_out[(dst_token_offsets[o]+t)*out_token_stride + h*head_dim + :] = out*
+ * dst_lse[h*dst_lse_head_stride + (dst_token_offsets[o]+t)*lse_token_stride] = lse*
+ * Math in fp32; out is stored in `dtype`, lse is fp32.  dst may alias one of
+ * the sources of the same op (in-place fold).  max_n_blocks_per_op <= 64.
+ */
+int dcp_update_out_lse(const void* src_out, void* dst_out,
+                       const float* src_lse, float* dst_lse, int n_head,
+                       const int32_t* src_block_table,
+                       const int32_t* dst_token_offsets,
+                       const int32_t* n_tokens_per_block,
+                       const int32_t* block_lengths, int n_red_ops,
+                       int block_size, int64_t out_block_stride,
+                       int64_t out_token_stride, int64_t lse_block_stride,
+                       int64_t lse_token_stride, int64_t src_lse_head_stride,
+                       int64_t dst_lse_head_stride, int head_dim,
+                       int max_n_blocks_per_op, int dtype, void* stream);
+
+/*
+ * N-way block sum (dQ / dK / dV accumulation) fused with the scatter.
+ * Replaces fused_blockwise_sum (fused_ops.py:1288-1360, kernels :1087-1285),
+ * called from _handle_sum (executor.py:1530-1545).
+ *   dst[s][dst_offsets[s]*dst_strides[s] + i] =
+ *       sum_{j < n_ops_per_block[s]} src[s][src_offsets[s*max_n+j]*src_strides[s] + i]
+ * for i < n_elements[s].  Accumulates in fp32 and rounds once (the reference
+ * kernel accumulates in the storage type; see its test tolerance 1e-2).
+ * dst may alias one of the sources of the same sum.
+ */
+int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_offsets,
+                      const int32_t* src_strides,
+                      const int32_t* n_ops_per_block, const int64_t* dst_ptrs,
+                      const int32_t* dst_offsets, const int32_t* dst_strides,
+                      const int32_t* n_elements, int n_sums,
+                      int max_n_ops_per_block, int64_t block_numel, int dtype,
+                      void* stream);
+
+/*
+ * Range-masked, paged, variable-length attention forward.
+ * Replaces dcp_flash_attn._flash_attn_varlen_forward as called by
+ * _wrapped_flash_attn_varlen_forward (executor.py:117-187) from _handle_attn
+ * (:884-913): no causal flag, no window, no dropout, no softcap.
+ *
+ * Batch row b = one q block.  Its seqlen_q = cu_seqlens_q[b+1]-cu_seqlens_q[b]
+ * (<= block_size) queries live in slot q_block_table[b] of `q`
+ * ([n_q_slots, block_size, n_heads_q, head_dim]); keys/values are the
+ * concatenation of slots kv_block_table[b*max_kv_blocks + j] of `k`/`v`
+ * (slot stride kv_slot_stride, token stride kv_token_stride, head stride
+ * head_dim, in elements) for kv positions [0, cu_seqlens_kv[b+1]-cu_seqlens_kv[b]).
+ * attn_range is int32 [n_ranges, 2, total_q]: query token t (global index
+ * cu_seqlens_q[b]+i) attends kv positions in the union of
+ * [attn_range[r][0][t], attn_range[r][1][t]).
+ * Writes out ([n_out_slots, block_size, n_heads_q, head_dim]) at slot
+ * out_block_table[b] and lse (fp32 [n_heads_q, n_out_slots, block_size]) at the
+ * same slot.  Rows with no visible key: out = 0, lse = +inf.
+ * q head h reads kv head h / (n_heads_q / n_heads_kv).
+ * row_order: optional device int32[batch], a permutation of the rows giving
+ * the order in which they are scheduled (put the rows with most keys first);
+ * NULL = as numbered.  It changes no result.
+ * Supported: dtype bf16/fp16, head_dim 64 or 128, block_size % 64 == 0,
+ * softmax_scale > 0.
+ */
+int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
+                 float* lse, const int32_t* cu_seqlens_q,
+                 const int32_t* cu_seqlens_kv, const int32_t* attn_range,
+                 int n_ranges, const int32_t* q_block_table,
+                 const int32_t* kv_block_table,
+                 const int32_t* out_block_table, const int32_t* row_order,
+                 int batch, int max_kv_blocks, int total_q, int block_size,
+                 int n_heads_q, int n_heads_kv, int head_dim,
+                 int64_t kv_slot_stride, int64_t kv_token_stride,
+                 int n_out_slots, float softmax_scale, int dtype,
+                 void* stream);
+
+/*
+ * Range-masked, paged, variable-length attention backward.
+ * Replaces dcp_flash_attn._flash_attn_varlen_backward as called by
+ * _wrapped_flash_attn_varlen_backward (executor.py:256-337) from
+ * _handle_attn_bw (:1058-1115).
+ *
+ * Inputs as dcp_attn_fwd plus dout/out (slots out_block_table[b]) and lse.
+ * dq ([n_dq_slots, block_size, n_heads_q, head_dim]) slot dq_block_table[b]
+ * receives the row's dQ.  dk/dv: slot dkv_block_table[b*max_kv_blocks + j]
+ * receives the dK/dV of the row's j-th kv block, summed over the q heads of
+ * each kv head's group; every token of that slot is written (tokens no query
+ * of the row attends get 0), so no pre-zeroing is needed.
+ * `dq_accum` is caller-provided fp32 scratch of total_q*n_heads_q*head_dim
+ * elements; `delta` fp32 scratch of total_q*n_heads_q.  Both are overwritten.
+ */
+int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+                 const void* out, const float* lse, void* dq, void* dk,
+                 void* dv, float* dq_accum, float* delta,
+                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_kv,
+                 const int32_t* attn_range, int n_ranges,
+                 const int32_t* q_block_table, const int32_t* kv_block_table,
+                 const int32_t* out_block_table,
+                 const int32_t* dq_block_table,
+                 const int32_t* dkv_block_table, int batch, int max_kv_blocks,
+                 int total_q, int block_size, int n_heads_q, int n_heads_kv,
+                 int head_dim, int64_t kv_slot_stride, int64_t kv_token_stride,
+                 int64_t dkv_slot_stride, int64_t dkv_token_stride,
+                 int n_out_slots, float softmax_scale, int dtype,
+                 void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DCP_HIP_H_ */

@@ -1,0 +1,89 @@
+"""Shared builders for plan-level tests: seeded inputs, the oracle run and the
+executor run of one synthetic single-device schedule."""
+
+import numpy as np
+import torch
+
+from dcp_amd.runtime.flash_attention.single_device import build_single_device_plans
+from dcp_amd.runtime.flash_attention.utils import MASK_FNS
+from oracle import dcp_oracle as oracle
+
+TORCH_DTYPE = {"bf16": torch.bfloat16, "fp16": torch.float16}
+
+
+def make_case(seqlens, block_size, n_heads, n_groups, head_dim, head_block, mask="causal",
+              mask_info=None, dtype="bf16", n_kv_groups=1, kv_split="round_robin", fold=False,
+              seed=0, qkv_scale=1.0, mask_kwargs=None):
+    mask_t = MASK_FNS[mask](list(seqlens), list(seqlens), torch.int32, mask_info, **(mask_kwargs or {}))
+    fw, bw, layout = build_single_device_plans(
+        seqlens, block_size, n_heads, n_groups, head_dim, head_block, mask_t,
+        dtype=TORCH_DTYPE[dtype], n_kv_groups=n_kv_groups, kv_split=kv_split, fold_stages=fold)
+    g = torch.Generator().manual_seed(seed)
+    T = sum(seqlens)
+    q = (torch.randn(T, n_heads, head_dim, generator=g) * qkv_scale).to(TORCH_DTYPE[dtype])
+    kv = (torch.randn(T, 2, n_groups, head_dim, generator=g) * qkv_scale).to(TORCH_DTYPE[dtype])
+    dout = torch.randn(T, n_heads, head_dim, generator=g).to(TORCH_DTYPE[dtype])
+    return dict(fw=fw, bw=bw, layout=layout, mask=mask_t, q=q, kv=kv, dout=dout, seqlens=list(seqlens),
+                head_block=head_block, head_dim=head_dim, dtype=dtype)
+
+
+def dense_truth(case, backward=False):
+    """Whole-sequence fp64 attention on the (already rounded) inputs."""
+    q = case["q"].float().numpy()
+    kv = case["kv"].float().numpy()
+    m = case["mask"].numpy()
+    if backward:
+        return oracle.dense_reference(q, kv, m, case["seqlens"], dout=case["dout"].float().numpy())
+    return oracle.dense_reference(q, kv, m, case["seqlens"])
+
+
+def run_executor(case, backward=False, use_graph=False, synchronous=False):
+    """Run the plans through the HIP executor.  Returns global-layout tensors
+    on the CPU: (out, lse) or (out, lse, dq, dkv)."""
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+
+    layout = case["layout"]
+    ex = get_executor(case["head_block"], case["head_dim"], None, fw_exec_plan=case["fw"],
+                      bw_exec_plan=case["bw"], synchronous=synchronous, use_cudagraph=use_graph)
+    ex.prepare(forward=True)
+    lq = layout.to_local_q(case["q"]).cuda()
+    lkv = layout.to_local_kv(case["kv"]).cuda()
+    if use_graph:
+        ex.init_forward_input(lq, lkv)
+        ex.execute(case["fw"], True)  # eager once
+        ex.capture_cudagraph()
+    out, lse = ex.forward(lq, lkv)
+    torch.cuda.synchronize()
+    res = [layout.from_local_q(out.cpu()), layout.from_local_lse(lse.cpu())]
+    if backward:
+        ex.switch_to_backward()
+        ldout = layout.to_local_q(case["dout"]).cuda()
+        if use_graph:
+            ex.capture_cudagraph()
+        dq, dkv = ex.backward(lq, lkv, out, ldout, lse)
+        torch.cuda.synchronize()
+        res += [layout.from_local_q(dq.cpu()), layout.from_local_kv(dkv.cpu())]
+    return res, ex
+
+
+def run_plan_oracle(case, backward=False):
+    layout = case["layout"]
+    po = oracle.PlanOracle(case["fw"], case["head_block"], case["head_dim"])
+    po.set("LocalQ", layout.to_local_q(case["q"]).float().numpy())
+    po.set("LocalKV", layout.to_local_kv(case["kv"]).float().numpy())
+    bufs = po.run()
+    out_l = torch.from_numpy(bufs["LocalOut"].copy())
+    lse_l = torch.from_numpy(bufs["LocalLSE"].copy())
+    res = [layout.from_local_q(out_l), layout.from_local_lse(lse_l)]
+    if backward:
+        pb = oracle.PlanOracle(case["bw"], case["head_block"], case["head_dim"])
+        pb.set("LocalQ", layout.to_local_q(case["q"]).float().numpy())
+        pb.set("LocalKV", layout.to_local_kv(case["kv"]).float().numpy())
+        pb.set("LocalOut", bufs["LocalOut"])
+        pb.buffers["LocalLSE"][...] = bufs["LocalLSE"]
+        pb.set("LocalOut", bufs["LocalOut"])
+        pb.set("LocaldOut", layout.to_local_q(case["dout"]).float().numpy())
+        b2 = pb.run()
+        res += [layout.from_local_q(torch.from_numpy(b2["LocaldQ"].copy())),
+                layout.from_local_kv(torch.from_numpy(b2["LocaldKV"].copy()))]
+    return res
