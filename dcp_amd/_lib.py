@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdcp_hip.so"
@@ -28,7 +28,8 @@ SIGNATURES = {
     "dcp_update_out_lse": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _L, _L, _L, _L, _L, _L, _I, _I, _I, _P],
     "dcp_blockwise_sum": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _P],
     "dcp_attn_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _F, _I, _P],
-    "dcp_attn_bwd": [_P] * 14 + [_I] + [_P] * 5 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
+    "dcp_attn_bwd": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
+    "dcp_attn_bwd_workspace_bytes": [_I, _I, _I, _I, _I],
 }
 
 _lock = threading.Lock()
@@ -56,7 +57,7 @@ def load():
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
-            fn.restype = c_char_p if name == "dcp_last_error" else c_int
+            fn.restype = {"dcp_last_error": c_char_p, "dcp_attn_bwd_workspace_bytes": c_size_t}.get(name, c_int)
         _lib = lib
     return _lib
 

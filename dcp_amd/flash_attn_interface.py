@@ -20,7 +20,17 @@ import torch
 from dcp_amd import _lib
 from dcp_amd.ops.fused_ops import dtype_code
 
-__all__ = ["_flash_attn_varlen_forward", "_flash_attn_varlen_backward"]
+__all__ = [
+    "_flash_attn_varlen_forward",
+    "_flash_attn_varlen_backward",
+    "backward_workspace_bytes",
+]
+
+
+def backward_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim) -> int:
+    """Scratch bytes ``_flash_attn_varlen_backward`` needs for these sizes."""
+    return int(_lib.load().dcp_attn_bwd_workspace_bytes(
+        int(batch), int(total_q), int(block_size), int(n_heads_q), int(head_dim)))
 
 
 def _stream() -> int:
@@ -175,8 +185,7 @@ def _flash_attn_varlen_backward(
     dq_block_table=None,
     dkv_block_table=None,
     rng_state=None,
-    dq_accum: Optional[torch.Tensor] = None,
-    delta: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None,
     row_order: Optional[torch.Tensor] = None,
 ):
     """Writes dQ into ``dq`` (slots ``dq_block_table``) and dK/dV into
@@ -185,9 +194,9 @@ def _flash_attn_varlen_backward(
     kernel, and every token of a dK/dV slot is written, so ``dk``/``dv`` need
     not be zeroed.
 
-    ``dq_accum`` (fp32, ``total_q * H * D`` elements) and ``delta`` (fp32,
-    ``total_q * H``) are scratch; pass preallocated tensors to keep the call
-    allocation-free (e.g. under graph capture), otherwise they are allocated
+    ``workspace`` is scratch of ``backward_workspace_bytes(...)`` bytes (any
+    dtype, contiguous); pass a preallocated tensor to keep the call
+    allocation-free (e.g. under graph capture), otherwise it is allocated
     here.
     """
     _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap, alibi_slopes)
@@ -212,20 +221,17 @@ def _flash_attn_varlen_backward(
         raise ValueError("dout and out must have the same number of slots")
     if softmax_scale is None:
         softmax_scale = head_dim ** (-0.5)
-    n_acc = int(total_q) * n_heads_q * head_dim
-    if dq_accum is None:
-        dq_accum = torch.empty(n_acc, dtype=torch.float32, device=q.device)
-    if delta is None:
-        delta = torch.empty(int(total_q) * n_heads_q, dtype=torch.float32, device=q.device)
-    if dq_accum.dtype != torch.float32 or dq_accum.numel() < n_acc:
-        raise ValueError("dq_accum must be float32 with total_q*H*D elements")
-    if delta.dtype != torch.float32 or delta.numel() < int(total_q) * n_heads_q:
-        raise ValueError("delta must be float32 with total_q*H elements")
+    need = backward_workspace_bytes(batch, int(total_q), block_size, n_heads_q, head_dim)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws_bytes = workspace.numel() * workspace.element_size()
+    if not workspace.is_contiguous() or ws_bytes < need:
+        raise ValueError(f"workspace must be contiguous with at least {need} bytes")
     _lib.call(
         "dcp_attn_bwd",
         dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
         softmax_lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-        dq_accum.data_ptr(), delta.data_ptr(),
+        workspace.data_ptr(), ws_bytes,
         _i32(cu_seqlens_q, "cu_seqlens_q").data_ptr(),
         _i32(cu_seqlens_k, "cu_seqlens_k").data_ptr(),
         attn_range.data_ptr(), n_ranges,
@@ -234,6 +240,7 @@ def _flash_attn_varlen_backward(
         _i32(out_block_table, "out_block_table").data_ptr(),
         _i32(dq_block_table, "dq_block_table").data_ptr(),
         _i32(dkv_block_table, "dkv_block_table").data_ptr(),
+        0 if row_order is None else _i32(row_order, "row_order").data_ptr(),
         batch, kv_block_table.shape[1], int(total_q), block_size,
         n_heads_q, n_heads_kv, head_dim,
         kv_slot_stride, kv_token_stride, dkv_slot_stride, dkv_token_stride,

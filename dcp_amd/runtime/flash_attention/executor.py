@@ -46,6 +46,7 @@ from dcp_amd.core.serialization import int_to_torch_dtype
 from dcp_amd.flash_attn_interface import (
     _flash_attn_varlen_backward,
     _flash_attn_varlen_forward,
+    backward_workspace_bytes,
 )
 from dcp_amd.ops.fused_ops import (
     flash_attn_update_out_lse,
@@ -392,6 +393,7 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
     total_q = sum(instr.seqlens_q)
     hb = exec.buffer_per_token_shape[BufferType.BUFFER_dQ][-2]
     d = exec.buffer_per_token_shape[BufferType.BUFFER_dQ][-1]
+    bs = exec.buffer_block_sizes[BufferType.BUFFER_dQ]
     exec._args_cache[exec.instr_index] = (
         total_q,
         sum(instr.seqlens_kv),
@@ -403,8 +405,11 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
         _mask_tensor(instr.attn_mask),
         _dev(_pad_block_table(instr.dq_block_table), torch.int32),
         _dev(_pad_block_table(instr.dkv_block_table), torch.int32),
-        torch.empty(total_q * hb * d, dtype=torch.float32, device="cuda"),  # dq accumulator
-        torch.empty(total_q * hb, dtype=torch.float32, device="cuda"),  # rowsum(dO*O)
+        torch.empty(
+            backward_workspace_bytes(len(instr.seqlens_q), total_q, bs, hb, d),
+            dtype=torch.uint8,
+            device="cuda",
+        ),
         _longest_first(instr.seqlens_kv),
     )
 
@@ -412,7 +417,7 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
 def _handle_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
     torch.cuda.nvtx.range_push("AttnBackwardInstr")
     (total_q, total_kv, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, dq_table, dkv_table,
-     dq_accum, delta, row_order) = exec._args_cache[exec.instr_index]
+     workspace, row_order) = exec._args_cache[exec.instr_index]
     k, v = _kv_views(exec.buffers[BufferType.BUFFER_KV])
     dk, dv = _kv_views(exec.buffers[BufferType.BUFFER_dKV])
     _flash_attn_varlen_backward(
@@ -445,8 +450,7 @@ def _handle_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
         out_block_table=out_table,
         dq_block_table=dq_table,
         dkv_block_table=dkv_table,
-        dq_accum=dq_accum,
-        delta=delta,
+        workspace=workspace,
         row_order=row_order,
     )
     torch.cuda.nvtx.range_pop()

@@ -19,6 +19,7 @@
 #ifndef DCP_HIP_H_
 #define DCP_HIP_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -189,24 +190,36 @@ int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
  * receives the row's dQ.  dk/dv: slot dkv_block_table[b*max_kv_blocks + j]
  * receives the dK/dV of the row's j-th kv block, summed over the q heads of
  * each kv head's group; every token of that slot is written (tokens no query
- * of the row attends get 0), so no pre-zeroing is needed.
- * `dq_accum` is caller-provided fp32 scratch of total_q*n_heads_q*head_dim
- * elements; `delta` fp32 scratch of total_q*n_heads_q.  Both are overwritten.
+ * of the row attends get 0), so no pre-zeroing is needed.  dQ is accumulated
+ * with fp32 atomics, so its last bits can differ from run to run.
+ * `workspace` is caller-provided device scratch of at least
+ * dcp_attn_bwd_workspace_bytes(...) bytes, 16-byte aligned; its contents are
+ * overwritten.  Key/value padding rows must hold finite values.
  */
 int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                  const void* out, const float* lse, void* dq, void* dk,
-                 void* dv, float* dq_accum, float* delta,
+                 void* dv, void* workspace, size_t workspace_bytes,
                  const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_kv,
                  const int32_t* attn_range, int n_ranges,
                  const int32_t* q_block_table, const int32_t* kv_block_table,
                  const int32_t* out_block_table,
                  const int32_t* dq_block_table,
-                 const int32_t* dkv_block_table, int batch, int max_kv_blocks,
-                 int total_q, int block_size, int n_heads_q, int n_heads_kv,
-                 int head_dim, int64_t kv_slot_stride, int64_t kv_token_stride,
+                 const int32_t* dkv_block_table, const int32_t* row_order,
+                 int batch, int max_kv_blocks, int total_q, int block_size,
+                 int n_heads_q, int n_heads_kv, int head_dim,
+                 int64_t kv_slot_stride, int64_t kv_token_stride,
                  int64_t dkv_slot_stride, int64_t dkv_token_stride,
                  int n_out_slots, float softmax_scale, int dtype,
                  void* stream);
+
+/*
+ * Bytes of scratch dcp_attn_bwd needs for these sizes: the fp32 dQ accumulator
+ * (total_q*n_heads_q*head_dim), rowsum(dO*O) (total_q*n_heads_q) and the
+ * per-(row, 64-query tile) range hulls.  No counterpart in the reference (its
+ * flash-attention fork allocates these inside the call).
+ */
+size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
+                                    int n_heads_q, int head_dim);
 
 #ifdef __cplusplus
 }
