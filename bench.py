@@ -1,0 +1,357 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-device blockwise attention path on one MI355X.
+
+One step = one forward plus one backward pass of the executor over a synthetic
+single-device block schedule (gather -> range-masked paged attention ->
+merge/scatter; gather -> attention backward -> block sums/scatter), with all
+inputs already resident in HBM and every argument table prepared, as the
+reference's micro-benchmark times only ``executor.execute(plan)``
+(benchmark/microbenchmark/benchmark_attention.py:976-1021).
+
+Prints ONE JSON line.  ``value`` is mask-aware attention TFLOP/s for fwd+bwd,
+with the reference cost model's FLOP convention (dcp/core/cost_model.py:120-127:
+fwd = 4*P*H*D, bwd = 2.5*fwd, P = unmasked (q, k) pairs).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
+
+
+# ---------------------------------------------------------------------------
+# workloads (BASELINE.json configs)
+# ---------------------------------------------------------------------------
+
+
+def lognormal_lengths(total, median, lo, hi, seed, sigma=1.0):
+    """Seeded lognormal sequence lengths that fill exactly ``total`` tokens."""
+    rng = np.random.default_rng(seed)
+    lengths, used = [], 0
+    while used < total:
+        n = int(np.clip(round(float(np.exp(rng.normal(np.log(median), sigma)))), lo, hi))
+        if total - used - n < lo:  # the remainder would be too short: take it all
+            n = total - used
+            if n > hi:
+                n = total - used - lo
+        lengths.append(n)
+        used += n
+    assert sum(lengths) == total and min(lengths) >= 1
+    return lengths
+
+
+def workload(name):
+    if name == "llama3_8b_causal_64k":
+        return dict(
+            seqlens=lognormal_lengths(65536, 4096, 256, 32768, seed=0),
+            block_size=1024, n_heads=32, n_groups=8, head_dim=128, head_block=4, mask="causal",
+            mask_info=None, mask_kwargs={},
+        )
+    if name == "lambda_128k":
+        return dict(
+            seqlens=lognormal_lengths(131072, 16384, 256, 65536, seed=0),
+            block_size=1024, n_heads=32, n_groups=8, head_dim=128, head_block=4, mask="lambda",
+            mask_info=None, mask_kwargs=dict(n_starting=64, l_pretrain=4096),
+        )
+    if name == "smoke":
+        return dict(
+            seqlens=[700, 300], block_size=256, n_heads=8, n_groups=2, head_dim=128, head_block=4,
+            mask="causal", mask_info=None, mask_kwargs={},
+        )
+    raise SystemExit(f"unknown workload {name}")
+
+
+def build(wl, backward=True):
+    import torch
+    from dcp_amd.runtime.flash_attention.single_device import build_single_device_plans
+    from dcp_amd.runtime.flash_attention.utils import MASK_FNS, count_attended_pairs
+
+    mask = MASK_FNS[wl["mask"]](wl["seqlens"], wl["seqlens"], torch.int32, wl["mask_info"], **wl["mask_kwargs"])
+    fw, bw, layout = build_single_device_plans(
+        wl["seqlens"], wl["block_size"], wl["n_heads"], wl["n_groups"], wl["head_dim"], wl["head_block"],
+        mask, dtype=torch.bfloat16, backward=backward)
+    pairs = count_attended_pairs(mask)
+    return fw, bw, layout, mask, pairs
+
+
+# ---------------------------------------------------------------------------
+# GPU side
+# ---------------------------------------------------------------------------
+
+
+def make_executors(wl, fw, bw, seed=0):
+    import torch
+    from dcp_amd.core.instructions import BufferType
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+
+    hb, d = wl["head_block"], wl["head_dim"]
+    ex_f = get_executor(hb, d, None, fw_exec_plan=fw, bw_exec_plan=bw)
+    ex_f.prepare(forward=True)
+    ex_b = get_executor(hb, d, None, fw_exec_plan=fw, bw_exec_plan=bw)
+    ex_b.mode = "Backward"
+    ex_b.prepare(forward=False)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    q = ex_f.buffers[BufferType.LOCAL_Q]
+    kv = ex_f.buffers[BufferType.LOCAL_KV]
+    q.copy_((torch.randn(q.shape, generator=g, device="cuda") * 0.5).to(q.dtype))
+    kv.copy_((torch.randn(kv.shape, generator=g, device="cuda") * 0.5).to(kv.dtype))
+    ex_f.execute(fw, True)
+    torch.cuda.synchronize()
+    ex_b.init_forward_input(q, kv)
+    ex_b.set_local_out_lse(ex_f.buffers[BufferType.LOCAL_OUT], ex_f.buffers[BufferType.LOCAL_LSE])
+    dout = ex_b.buffers[BufferType.LOCAL_dOUT]
+    dout.copy_(torch.randn(dout.shape, generator=g, device="cuda").to(dout.dtype))
+    return ex_f, ex_b
+
+
+def step(ex_f, ex_b, fw, bw):
+    ex_f.execute(fw, True)
+    ex_b.execute(bw, False)
+
+
+def time_steps(ex_f, ex_b, fw, bw, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        step(ex_f, ex_b, fw, bw)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(ex_f, ex_b, fw, bw)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def kernel_times(ex_f, ex_b, fw, bw, steps):
+    """Average duration of every kernel of the library over ``steps`` steps,
+    from events recorded on the launch stream by the library itself."""
+    import torch
+    from dcp_amd import _lib
+
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    for _ in range(steps):
+        step(ex_f, ex_b, fw, bw)
+    torch.cuda.synchronize()
+    _lib.profile_enable(False)
+    rep = _lib.profile_report()
+    return {name: dict(launches=n, avg_ms=total / n, ms_per_step=total / steps) for name, (n, total) in rep.items()}
+
+
+def movement_microbench(iters=5):
+    """BASELINE config 5: 262144 tokens x 32 heads x 128, bf16, 512-token
+    blocks; gather through a seeded block permutation, inverse scatter, then a
+    4-way (out, lse) merge.  Returns GB/s from events on the launch stream."""
+    import torch
+    from dcp_amd import _lib
+    from dcp_amd.ops.fused_ops import flash_attn_update_out_lse, fused_copy_bf16_varlen
+
+    tokens, heads, d, bs = 262144, 32, 128, 512
+    n_blocks = tokens // bs
+    numel = bs * heads * d
+    rng = np.random.default_rng(0)
+    perm = rng.permutation(n_blocks)
+    src = torch.randn(tokens, heads, d, device="cuda", dtype=torch.bfloat16)
+    packed = torch.empty_like(src)
+    back = torch.empty_like(src)
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    i32 = lambda v: torch.tensor(np.asarray(v), dtype=torch.int32, device="cuda")
+    ident = np.arange(n_blocks)
+    full = i32([numel] * n_blocks)
+    stride = i32([numel] * n_blocks)
+    gather = (i64([src.data_ptr()] * n_blocks), i32(ident), stride, i64([packed.data_ptr()] * n_blocks), i32(perm), stride, full)
+    scatter = (i64([packed.data_ptr()] * n_blocks), i32(perm), stride, i64([back.data_ptr()] * n_blocks), i32(ident), stride, full)
+    fused_copy_bf16_varlen(*gather, numel, 128)
+    fused_copy_bf16_varlen(*scatter, numel, 128)
+    torch.cuda.synchronize()
+    exact = bool(torch.equal(back, src))
+    _lib.profile_enable(True)
+    for _ in range(iters):
+        fused_copy_bf16_varlen(*gather, numel, 128)
+        fused_copy_bf16_varlen(*scatter, numel, 128)
+    torch.cuda.synchronize()
+    _lib.profile_enable(False)
+    n, total = _lib.profile_report()["copy_varlen_kernel"]
+    copy_bytes = 2 * tokens * heads * d * 2
+    copy_gbps = copy_bytes / (total / n * 1e-3) / 1e9
+    del packed, back
+
+    # merge: 4 partial outs per q block
+    n_src = 4
+    outs = torch.randn(n_src * n_blocks, bs, heads, d, device="cuda", dtype=torch.bfloat16)
+    lses = torch.rand(heads, n_src * n_blocks, bs, device="cuda") * 10 - 5
+    dst_out = torch.empty(tokens, heads, d, device="cuda", dtype=torch.bfloat16)
+    dst_lse = torch.empty(heads, tokens, device="cuda")
+    table = i32(rng.permutation(n_src * n_blocks).reshape(n_blocks, n_src))
+    args = (outs, dst_out, lses, dst_lse, heads, table, i32(ident * bs), i32([bs] * n_blocks), i32([n_src] * n_blocks),
+            bs, numel, heads * d, bs, 1, n_src * n_blocks * bs, tokens, d, n_src, 64)
+    flash_attn_update_out_lse(*args)
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    for _ in range(iters):
+        flash_attn_update_out_lse(*args)
+    torch.cuda.synchronize()
+    _lib.profile_enable(False)
+    n, total = _lib.profile_report()["merge_out_lse_kernel"]
+    merge_bytes = (n_src + 1) * (d * 2 + 4) * tokens * heads
+    merge_gbps = merge_bytes / (total / n * 1e-3) / 1e9
+    return dict(
+        workload="block movement: 262144 tok x 32 heads x 128 bf16, 512-token blocks, seeded permutation",
+        gather_scatter_GBps=round(copy_gbps, 1),
+        gather_scatter_frac_of_8TBps=round(copy_gbps / PEAK_HBM_GBPS, 4),
+        gather_scatter_roundtrip_bit_exact=exact,
+        copy_bytes_per_launch=copy_bytes,
+        merge4_GBps=round(merge_gbps, 1),
+        merge4_frac_of_8TBps=round(merge_gbps / PEAK_HBM_GBPS, 4),
+        merge_bytes_per_launch=merge_bytes,
+    )
+
+
+# ---------------------------------------------------------------------------
+# CPU baseline: the oracle on a bounded, seeded sample of q-block rows
+# ---------------------------------------------------------------------------
+
+
+def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
+    """Times the numpy oracle's fwd+bwd of whole q-block rows (all heads of the
+    row's head block) drawn from the workload's backward plan until about
+    ``budget_s`` seconds of CPU work are done."""
+    from oracle import dcp_oracle as oracle
+
+    try:
+        from threadpoolctl import threadpool_info
+
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = 1
+    instr = next(i for i in fw.instructions if type(i).__name__ == "AttnInstr")
+    mask = np.asarray(instr.attn_mask)
+    if mask.ndim == 2:
+        mask = mask[None]
+    rng = np.random.default_rng(seed)
+    order = rng.permutation(len(instr.seqlens_q))
+    hb, d, bs = wl["head_block"], wl["head_dim"], wl["block_size"]
+    hkv = max(1, hb // (wl["n_heads"] // wl["n_groups"]))
+    cu = np.concatenate(([0], np.cumsum(instr.seqlens_q)))
+    pairs, rows, elapsed = 0, 0, 0.0
+    for b in order:
+        n_kv = instr.seqlens_kv[b]
+        q = (rng.standard_normal((bs, hb, d)) * 0.5).astype(np.float32)
+        k = (rng.standard_normal((n_kv, hkv, d)) * 0.5).astype(np.float32)
+        v = (rng.standard_normal((n_kv, hkv, d)) * 0.5).astype(np.float32)
+        dout = rng.standard_normal((bs, hb, d)).astype(np.float32)
+        allowed = oracle.ranges_to_bool(mask[:, :, cu[b] : cu[b + 1]], n_kv)
+        t0 = time.perf_counter()
+        out, lse = oracle.range_attention_fwd(q, k, v, allowed, dtype=np.float32)
+        oracle.range_attention_bwd(q, k, v, out, lse, dout, allowed, dtype=np.float32)
+        elapsed += time.perf_counter() - t0
+        pairs += int(allowed.sum())
+        rows += 1
+        if elapsed >= budget_s:
+            break
+    flops = oracle.attention_flops(pairs, hb, d, "fwd+bwd")
+    return dict(
+        value=round(flops / elapsed / 1e12, 5), unit="TFLOP/s", cores=int(threads), kind="port",
+        sample=f"{rows} seeded q-block rows of the same schedule (fwd+bwd, fp32 numpy oracle, {elapsed:.1f} s)",
+    )
+
+
+# ---------------------------------------------------------------------------
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama3_8b_causal_64k")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-movement", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit(
+            "bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible")
+    from dcp_amd import _lib
+
+    _lib.load()
+    torch.cuda.set_device(0)
+    wl = workload(args.workload)
+    fw, bw, layout, mask, pairs = build(wl)
+    flops_fwd = 4.0 * pairs * wl["n_heads"] * wl["head_dim"]
+    flops_step = 3.5 * flops_fwd
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(wl, fw, bw, budget_s=args.cpu_seconds)
+
+    ex_f, ex_b = make_executors(wl, fw, bw)
+    sec = time_steps(ex_f, ex_b, fw, bw, args.steps, args.warmup)
+    kt = kernel_times(ex_f, ex_b, fw, bw, max(2, min(args.steps, 5)))
+    value = flops_step / sec / 1e12
+
+    bwd = kt["attn_bwd_kernel"]
+    fwd = kt["attn_fwd_kernel"]
+    bwd_tflops = 2.5 * flops_fwd / (bwd["avg_ms"] * 1e-3) / 1e12
+    fwd_tflops = flops_fwd / (fwd["avg_ms"] * 1e-3) / 1e12
+    roofline = dict(
+        bound="mfma", kernel="attn_bwd_kernel", achieved=round(bwd_tflops, 2), peak=PEAK_BF16_TFLOPS,
+        unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4), traffic=None,
+        flops_per_launch=2.5 * flops_fwd, avg_launch_ms=round(bwd["avg_ms"], 4),
+    )
+    extra = dict(
+        attn_fwd_kernel=dict(achieved_TFLOPs=round(fwd_tflops, 2), frac_of_peak=round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
+                             avg_launch_ms=round(fwd["avg_ms"], 4)),
+        kernel_ms_per_step={k: round(v["ms_per_step"], 4) for k, v in sorted(kt.items())},
+    )
+    if not args.no_movement:
+        del ex_f, ex_b
+        torch.cuda.empty_cache()
+        extra["block_movement"] = movement_microbench()
+
+    line = {
+        "metric": "mask-aware attn fwd+bwd TFLOP/s @1 MI355X; block merge/gather HBM GB/s",
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload,
+            "tokens": int(sum(wl["seqlens"])), "n_sequences": len(wl["seqlens"]),
+            "max_seqlen": int(max(wl["seqlens"])), "block_size": wl["block_size"],
+            "q_heads": wl["n_heads"], "kv_heads": wl["n_groups"], "head_dim": wl["head_dim"],
+            "head_block": wl["head_block"], "mask": wl["mask"], "unmasked_pairs_per_head": int(pairs),
+            "flops_per_step": flops_step,
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -22,6 +22,8 @@ _F = c_float
 SIGNATURES = {
     "dcp_version": [],
     "dcp_last_error": [],
+    "dcp_profile_enable": [_I],
+    "dcp_profile_report": [c_char_p, c_size_t],
     "dcp_fused_copy_varlen": [_P, _P, _P, _P, _P, _P, _P, _I, _L, _I, _P],
     "dcp_fused_copy_varlen_dkv": [_P, _P, _P, _I, _I, _I, _I, _P],
     "dcp_fused_copy_varlen_lse": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
@@ -60,6 +62,24 @@ def load():
             fn.restype = {"dcp_last_error": c_char_p, "dcp_attn_bwd_workspace_bytes": c_size_t}.get(name, c_int)
         _lib = lib
     return _lib
+
+
+def profile_enable(on: bool) -> None:
+    load().dcp_profile_enable(1 if on else 0)
+
+
+def profile_report() -> dict:
+    """``{kernel name: (launches, total milliseconds)}`` of the launches made
+    while profiling was enabled; clears the record."""
+    buf = ctypes.create_string_buffer(1 << 16)
+    status = load().dcp_profile_report(buf, len(buf))
+    if status != 0:
+        raise DcpHipError("dcp_profile_report: buffer too small")
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, count, total = line.rsplit(" ", 2)
+        out[name] = (int(count), float(total))
+    return out
 
 
 def last_error() -> str:

@@ -1,13 +1,77 @@
-// Version and error-string entry points of libdcp_hip.so.
+// Version, error-string and profiling entry points of libdcp_hip.so.
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
 #include "common.h"
 
 namespace dcp {
+
 char* last_error_buffer() {
   static thread_local char buffer[512] = {0};
   return buffer;
 }
+
+namespace {
+struct Span {
+  std::string name;
+  hipEvent_t start, stop;
+};
+std::mutex g_mu;
+bool g_profiling = false;
+std::vector<Span> g_spans;
+}  // namespace
+
+bool profiling_enabled() { return g_profiling; }
+
+void profile_begin(const char* name, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  Span s;
+  s.name = name;
+  if (hipEventCreate(&s.start) != hipSuccess || hipEventCreate(&s.stop) != hipSuccess) return;
+  (void)hipEventRecord(s.start, stream);
+  g_spans.push_back(s);
+}
+
+void profile_end(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_spans.empty()) (void)hipEventRecord(g_spans.back().stop, stream);
+}
+
 }  // namespace dcp
 
 extern "C" int dcp_version(void) { return 100; }
 
 extern "C" const char* dcp_last_error(void) { return dcp::last_error_buffer(); }
+
+extern "C" void dcp_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(dcp::g_mu);
+  dcp::g_profiling = on != 0;
+}
+
+extern "C" int dcp_profile_report(char* buffer, size_t capacity) {
+  std::lock_guard<std::mutex> lock(dcp::g_mu);
+  std::map<std::string, std::pair<double, long>> totals;
+  for (auto& s : dcp::g_spans) {
+    float ms = 0.0f;
+    if (hipEventSynchronize(s.stop) == hipSuccess && hipEventElapsedTime(&ms, s.start, s.stop) == hipSuccess) {
+      auto& t = totals[s.name];
+      t.first += ms;
+      t.second += 1;
+    }
+    (void)hipEventDestroy(s.start);
+    (void)hipEventDestroy(s.stop);
+  }
+  dcp::g_spans.clear();
+  std::string text;
+  char line[256];
+  for (auto& kv : totals) {
+    snprintf(line, sizeof line, "%s %ld %.6f\n", kv.first.c_str(), kv.second.second, kv.second.first);
+    text += line;
+  }
+  if (buffer && capacity > 0) {
+    snprintf(buffer, capacity, "%s", text.c_str());
+  }
+  return (int)text.size() < (int)capacity ? DCP_OK : DCP_ERR_ARG;
+}

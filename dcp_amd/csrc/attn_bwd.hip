@@ -500,12 +500,24 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t stream) {
   const int64_t chunks = (rows + ROWS - 1) / ROWS;
   DCP_REQUIRE(chunks <= 65535, "attn_bwd: block of %lld (token, head) rows is too large", (long long)rows);
   dim3 prep_grid(p.batch, (unsigned)chunks);
-  hipLaunchKernelGGL((bwd_prep_kernel<DTYPE, D>), prep_grid, dim3(256), 0, stream, p);
-  hipLaunchKernelGGL(bwd_tile_hull_kernel, dim3(p.batch * p.q_tiles_per_row), dim3(64), 0, stream, p);
+  {
+    KernelTimer timer("bwd_prep_kernel", stream);
+    hipLaunchKernelGGL((bwd_prep_kernel<DTYPE, D>), prep_grid, dim3(256), 0, stream, p);
+  }
+  {
+    KernelTimer timer("bwd_tile_hull_kernel", stream);
+    hipLaunchKernelGGL(bwd_tile_hull_kernel, dim3(p.batch * p.q_tiles_per_row), dim3(64), 0, stream, p);
+  }
   const int64_t n_wg = (int64_t)p.batch * p.n_heads_kv * p.kv_tiles_per_row;
   DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_bwd: grid too large");
-  hipLaunchKernelGGL((attn_bwd_kernel<DTYPE, D>), dim3((unsigned)n_wg), dim3(kBwdThreads), 0, stream, p);
-  hipLaunchKernelGGL((bwd_dq_store_kernel<DTYPE, D>), prep_grid, dim3(256), 0, stream, p);
+  {
+    KernelTimer timer("attn_bwd_kernel", stream);
+    hipLaunchKernelGGL((attn_bwd_kernel<DTYPE, D>), dim3((unsigned)n_wg), dim3(kBwdThreads), 0, stream, p);
+  }
+  {
+    KernelTimer timer("bwd_dq_store_kernel", stream);
+    hipLaunchKernelGGL((bwd_dq_store_kernel<DTYPE, D>), prep_grid, dim3(256), 0, stream, p);
+  }
   return check_launch("attn_bwd kernels");
 }
 

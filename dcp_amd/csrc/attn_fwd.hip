@@ -376,6 +376,7 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   const int64_t n_wg = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
   DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_fwd: grid too large");
   dim3 grid((unsigned)n_wg), block(kFwdThreads);
+  KernelTimer timer("attn_fwd_kernel", stream);
 #define DCP_FWD(DT, HD) \
   hipLaunchKernelGGL((attn_fwd_kernel<DT, HD>), grid, block, 0, (hipStream_t)stream, p)
   if (dtype == DCP_DTYPE_BF16) {

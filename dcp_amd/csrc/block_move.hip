@@ -100,6 +100,7 @@ static int launch_copy(const int64_t* src_ptrs, const int32_t* src_offsets,
   const int64_t chunks = (block_bytes + kCopyChunkBytes - 1) / kCopyChunkBytes;
   DCP_REQUIRE(chunks * n_ptrs < (int64_t)1 << 31, "copy grid too large: %lld blocks x %lld chunks",
               (long long)n_ptrs, (long long)chunks);
+  KernelTimer timer("copy_varlen_kernel", stream);
   hipLaunchKernelGGL(copy_varlen_kernel, dim3((unsigned)(chunks * n_ptrs)), dim3(kCopyThreads), 0,
                      (hipStream_t)stream, src_ptrs, src_offsets, src_strides, dst_ptrs,
                      dst_offsets, dst_strides, n_count, elems_per_count, (int)chunks, elem_size);
@@ -157,6 +158,7 @@ extern "C" int dcp_fused_copy_varlen_lse(const int64_t* src_ptrs,
                   dst_token_offsets && dst_head_strides && n_tokens,
               "lse copy: null table");
   dim3 grid(n_ptrs, head_block_size, (max_n_tokens + 255) / 256);
+  KernelTimer timer("copy_lse_kernel", stream);
   if (elem_size == 4)
     hipLaunchKernelGGL(copy_lse_kernel<uint32_t>, grid, dim3(256), 0, (hipStream_t)stream,
                        src_ptrs, src_token_offsets, src_head_strides, dst_ptrs, dst_token_offsets,

@@ -151,6 +151,7 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
   DCP_REQUIRE(row_chunks <= 65535, "merge: block of %lld (token, head) rows is too large",
               (long long)rows);
   dim3 grid(n_red_ops, (unsigned)row_chunks);
+  KernelTimer timer("merge_out_lse_kernel", stream);
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(256), 0, (hipStream_t)stream, (const raw*)src_out,
                        (raw*)dst_out, src_lse, dst_lse, n_head, src_block_table,
@@ -276,6 +277,7 @@ extern "C" int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_off
   const int64_t chunks = (block_numel + chunk_elems - 1) / chunk_elems;
   DCP_REQUIRE(chunks <= 65535, "sum: block of %lld elements is too large", (long long)block_numel);
   dim3 grid(n_sums, (unsigned)chunks);
+  KernelTimer timer("blockwise_sum_kernel", stream);
 #define DCP_SUM_LAUNCH(DT)                                                                     \
   hipLaunchKernelGGL(blockwise_sum_kernel<DT>, grid, dim3(256), 0, (hipStream_t)stream,        \
                      src_ptrs, src_offsets, src_strides, n_ops_per_block, dst_ptrs,            \

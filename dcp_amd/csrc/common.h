@@ -33,6 +33,26 @@ inline int check_launch(const char* what) {
     if (!(cond)) return ::dcp::fail(DCP_ERR_ARG, __VA_ARGS__); \
   } while (0)
 
+// ---- optional per-kernel timing (off by default) -----------------------------
+// While enabled through dcp_profile_enable(1), every kernel launch is bracketed
+// by two events recorded on the launch stream; dcp_profile_report() waits for
+// them and sums the elapsed time per kernel name.  Nothing is recorded, created
+// or synchronised when profiling is off.
+bool profiling_enabled();
+void profile_begin(const char* name, hipStream_t stream);
+void profile_end(hipStream_t stream);
+
+struct KernelTimer {
+  hipStream_t stream;
+  bool on;
+  KernelTimer(const char* name, void* s) : stream((hipStream_t)s), on(profiling_enabled()) {
+    if (on) profile_begin(name, stream);
+  }
+  ~KernelTimer() {
+    if (on) profile_end(stream);
+  }
+};
+
 // ---- 16-byte vector --------------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

@@ -42,6 +42,18 @@ int dcp_version(void);
 const char* dcp_last_error(void);
 
 /*
+ * Per-kernel timing for benchmarks (no counterpart in the reference, which
+ * relies on external profilers).  While enabled, each kernel launch of this
+ * library is bracketed by two events recorded on its launch stream.
+ * dcp_profile_report waits for the recorded events, writes one line per kernel
+ * name, "<name> <launches> <total_ms>\n", into `buffer` (NUL-terminated) and
+ * forgets them; it returns nonzero if `capacity` was too small.  Disabled (the
+ * default), launches record nothing.
+ */
+void dcp_profile_enable(int on);
+int dcp_profile_report(char* buffer, size_t capacity);
+
+/*
  * Block gather / scatter through pointer tables.
  * Replaces dcp.ops.fused_ops.fused_copy_{bf16,fp16,fp32}_varlen
  * (dcp/ops/fused_ops.py:842-864, 916-938, 1013-1035; kernels :290-335,
