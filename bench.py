@@ -306,18 +306,25 @@ def main():
     kt = kernel_times(ex_f, ex_b, fw, bw, max(2, min(args.steps, 5)))
     value = flops_step / sec / 1e12
 
-    bwd = kt["attn_bwd_kernel"]
-    fwd = kt["attn_fwd_kernel"]
-    bwd_tflops = 2.5 * flops_fwd / (bwd["avg_ms"] * 1e-3) / 1e12
+    # The backward is two kernels (dK/dV key-outer, dQ query-outer) that together do
+    # the algorithmic backward work 2.5 * fwd; they are priced as one unit.
+    dkv, dq, fwd = kt["attn_bwd_dkv_kernel"], kt["attn_bwd_dq_kernel"], kt["attn_fwd_kernel"]
+    bwd_ms = dkv["avg_ms"] + dq["avg_ms"]
+    bwd_tflops = 2.5 * flops_fwd / (bwd_ms * 1e-3) / 1e12
     fwd_tflops = flops_fwd / (fwd["avg_ms"] * 1e-3) / 1e12
     roofline = dict(
-        bound="mfma", kernel="attn_bwd_kernel", achieved=round(bwd_tflops, 2), peak=PEAK_BF16_TFLOPS,
-        unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4), traffic=None,
-        flops_per_launch=2.5 * flops_fwd, avg_launch_ms=round(bwd["avg_ms"], 4),
+        bound="mfma", kernel="attn_bwd_dkv_kernel+attn_bwd_dq_kernel", achieved=round(bwd_tflops, 2),
+        peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4), traffic=None,
+        flops_per_launch=2.5 * flops_fwd, avg_launch_ms=round(bwd_ms, 4),
     )
     extra = dict(
         attn_fwd_kernel=dict(achieved_TFLOPs=round(fwd_tflops, 2), frac_of_peak=round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
                              avg_launch_ms=round(fwd["avg_ms"], 4)),
+        # executed MFMA work: dK/dV kernel 4 products (S, dP, dV, dK), dQ kernel 3 (S, dP, dQ)
+        attn_bwd_dkv_kernel=dict(executed_TFLOPs=round(2.0 * flops_fwd / (dkv["avg_ms"] * 1e-3) / 1e12, 2),
+                                 avg_launch_ms=round(dkv["avg_ms"], 4)),
+        attn_bwd_dq_kernel=dict(executed_TFLOPs=round(1.5 * flops_fwd / (dq["avg_ms"] * 1e-3) / 1e12, 2),
+                                avg_launch_ms=round(dq["avg_ms"], 4)),
         kernel_ms_per_step={k: round(v["ms_per_step"], 4) for k, v in sorted(kt.items())},
     )
     if not args.no_movement:

@@ -7,11 +7,12 @@ every operator raises instead of falling back to another implementation.
 from __future__ import annotations
 
 import ctypes
+import os
 import threading
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libdcp_hip.so"
+LIB_PATH = Path(os.environ.get("DCP_LIB_PATH", Path(__file__).resolve().parent / "libdcp_hip.so"))
 
 _P = c_void_p
 _I = c_int
@@ -55,6 +56,11 @@ def load():
                 f"{LIB_PATH} is not built; run `python -m dcp_amd.build` "
                 "(there is no fallback implementation)"
             )
+        # torch bundles its own HIP runtime (same soname as the system one).
+        # It must be in the process before this library is, so that both bind
+        # to one runtime; two runtimes in one process do not share a device.
+        import torch  # noqa: F401
+
         lib = ctypes.CDLL(str(LIB_PATH))
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)

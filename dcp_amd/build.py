@@ -16,7 +16,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 INCLUDE = PKG_DIR.parent / "include"
-LIB_PATH = PKG_DIR / "libdcp_hip.so"
+LIB_PATH = Path(os.environ.get("DCP_LIB_PATH", PKG_DIR / "libdcp_hip.so"))
 BUILD_DIR = PKG_DIR / "csrc" / "build"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -35,6 +35,10 @@ FLAGS = [
     "-Xclang",
     "-packed-fp32-ops",
 ]
+
+
+# extra compiler flags for experiments, e.g. DCP_EXTRA_HIPCC_FLAGS="-DFOO=1"
+FLAGS += os.environ.get("DCP_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def sources():

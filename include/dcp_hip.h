@@ -202,8 +202,8 @@ int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
  * receives the row's dQ.  dk/dv: slot dkv_block_table[b*max_kv_blocks + j]
  * receives the dK/dV of the row's j-th kv block, summed over the q heads of
  * each kv head's group; every token of that slot is written (tokens no query
- * of the row attends get 0), so no pre-zeroing is needed.  dQ is accumulated
- * with fp32 atomics, so its last bits can differ from run to run.
+ * of the row attends get 0), so no pre-zeroing is needed.  No atomics are
+ * used: results are bit-reproducible from run to run.
  * `workspace` is caller-provided device scratch of at least
  * dcp_attn_bwd_workspace_bytes(...) bytes, 16-byte aligned; its contents are
  * overwritten.  Key/value padding rows must hold finite values.
@@ -225,9 +225,8 @@ int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                  void* stream);
 
 /*
- * Bytes of scratch dcp_attn_bwd needs for these sizes: the fp32 dQ accumulator
- * (total_q*n_heads_q*head_dim), rowsum(dO*O) (total_q*n_heads_q) and the
- * per-(row, 64-query tile) range hulls.  No counterpart in the reference (its
+ * Bytes of scratch dcp_attn_bwd needs for these sizes: rowsum(dO*O)
+ * (total_q*n_heads_q floats) and the per-(row, 64-query tile) range hulls.  No counterpart in the reference (its
  * flash-attention fork allocates these inside the call).
  */
 size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
