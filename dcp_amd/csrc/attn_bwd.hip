@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         float pv[4], dsv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float e = exp2f(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));
+          float e = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));
           float ds = e * (dp_acc[4 * g + r] - d4[r]);
           if (!unmasked) {
             const int4 rg = *reinterpret_cast<const int4*>(&rng_lds[(qrow + r) * 4]);
@@ -581,7 +581,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int i = g * 8 + j;
-          float pr = exp2f(fmaf(s_acc[i], p.scale_log2, -lse2));
+          float pr = fast_exp2(fmaf(s_acc[i], p.scale_log2, -lse2));
           float ds = pr * (dp_acc[i] - delta);
           if (!unmasked) ds = rng.contains(kb + 8 * (i / 4) + (i % 4)) ? ds : 0.0f;
           e[j] = ds;

@@ -14,6 +14,13 @@
 // rescale factor is a per-lane scalar, and the masked range of the row lives
 // in four registers.
 //
+// K and V tiles go from global memory straight into LDS (global_load_lds, no
+// register staging), in two stages: the next tile streams in while the current
+// one is multiplied.  The row order and padding of each tile are chosen so that
+// operand reads are conflict-free and every LDS address in the key loop is a
+// per-lane base plus an immediate.  V^T is never materialised: the transposing
+// LDS load delivers it from the V tile.
+//
 // Key tiles are chosen per workgroup from the hull of its rows' ranges (tiles
 // no row can see are never loaded), each wave skips tiles outside its own
 // rows' hull, and a tile that lies inside every row's range of the wave skips
@@ -58,12 +65,16 @@ constexpr int kFwdThreads = 256;
 template <int DTYPE, int D>
 __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdParams p) {
   constexpr int BN = kFwdBN;
-  constexpr int KS = D / 16;         // k-steps of S^T = K Q^T
-  constexpr int DT = D / 32;         // 32-row tiles of O^T
-  constexpr int K_STRIDE = D + 8;    // elements; 16-byte reads of 16 lanes hit 64 distinct banks
-  constexpr int VT_STRIDE = BN + 8;  // elements
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[BN * K_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[D * VT_STRIDE];
+  constexpr int KS = D / 16;  // k-steps of S^T = K Q^T
+  constexpr int DT = D / 32;  // 32-row tiles of O^T
+  typedef RowTile<D> KTile;  // read as rows (A operand of S^T)
+  typedef ColTile<D> VTile;  // read as columns (A operand of O^T = V^T P^T)
+  // two stages of (K tile, V tile); separate arrays so the compiler can tell
+  // the stage being filled from the stage being read
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds0[KTile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds0[VTile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds1[KTile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds1[VTile::SIZE];
   __shared__ int hull_lds[4][4];
 
   const int tid = threadIdx.x;
@@ -140,8 +151,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
     g_lo1 = min(g_lo1, hull_lds[i][2]);
     g_hi1 = max(g_hi1, hull_lds[i][3]);
   }
-  const int kt_begin = min(g_lo0, g_lo1) / BN;
-  const int kt_end = (max(g_hi0, g_hi1) + BN - 1) / BN;  // 0 when nothing is visible
+  const TileRuns runs(g_lo0, g_hi0, g_lo1, g_hi1, BN);
+  const int n_tiles = runs.count();
 
   // ---- running state ---------------------------------------------------------
   f32x16 o_acc[DT];
@@ -156,108 +167,81 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
   const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
 
-  // global -> LDS staging maps
-  constexpr int CH = D / 8;                    // 16-byte chunks per row
-  constexpr int K_ROWS_PER_PASS = kFwdThreads / CH;
-  constexpr int K_PASSES = BN / K_ROWS_PER_PASS;
-  constexpr int V_UNITS = (BN / 4) * CH;       // (4 keys) x (8 dims) units
-  constexpr int V_PASSES = (V_UNITS + kFwdThreads - 1) / kFwdThreads;
-  const int k_row = tid / CH, k_chunk = tid % CH;
+  // loop-invariant per-lane pieces of every address used in the key loop
+  uint32_t k_goff[KTile::LPW], v_goff[VTile::LPW];
+  KTile::lane_offsets(k_goff, p.kv_token_stride, w, lane);
+  VTile::lane_offsets(v_goff, p.kv_token_stride, w, lane);
+  const int k_rd = KTile::at(c, 8 * h);         // + nt*32 rows, + ks*16 elements
+  const int v_rd = VTile::lane_base(lane, true);  // + slot / column block offsets
 
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
+  // fill one stage with key tile `kt`
+  auto fetch = [&](int kt, uint16_t* k_dst, uint16_t* v_dst) {
     const int k0 = kt * BN;
-    const bool wg_active = (k0 < g_hi0 && k0 + BN > g_lo0) || (k0 < g_hi1 && k0 + BN > g_lo1);
-    if (!wg_active) continue;
-
-    // ---- stage K (row-major) and V (transposed, k-slot order) into LDS ------
     const int blk = k0 / p.block_size;
-    const int tok0 = k0 - blk * p.block_size;
-    const int64_t tile_off = (int64_t)kv_table[blk] * p.kv_slot_stride + (int64_t)tok0 * p.kv_token_stride;
-    u32x4 kst[K_PASSES];
-#pragma unroll
-    for (int ps = 0; ps < K_PASSES; ++ps) {
-      const int r = ps * K_ROWS_PER_PASS + k_row;
-      kst[ps] = *reinterpret_cast<const u32x4*>(kg + tile_off + (int64_t)r * p.kv_token_stride + k_chunk * 8);
-    }
-    u32x4 vst[V_PASSES][4];
-#pragma unroll
-    for (int ps = 0; ps < V_PASSES; ++ps) {
-      const int u = ps * kFwdThreads + tid;
-      if (u < V_UNITS) {
-        const int kvg = u % (BN / 4), dg = u / (BN / 4);
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          vst[ps][r] = *reinterpret_cast<const u32x4*>(
-              vg + tile_off + (int64_t)(kvg * 4 + r) * p.kv_token_stride + dg * 8);
-      }
-    }
-    __syncthreads();  // everyone is done reading the previous tile
-#pragma unroll
-    for (int ps = 0; ps < K_PASSES; ++ps) {
-      const int r = ps * K_ROWS_PER_PASS + k_row;
-      *reinterpret_cast<u32x4*>(&k_lds[r * K_STRIDE + k_chunk * 8]) = kst[ps];
-    }
-#pragma unroll
-    for (int ps = 0; ps < V_PASSES; ++ps) {
-      const int u = ps * kFwdThreads + tid;
-      if (u < V_UNITS) {
-        const int kvg = u % (BN / 4), dg = u / (BN / 4);
-        const int pos = (kvg / 4) * 16 + kslot_pos(kvg % 4);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          const uint32_t a0 = vst[ps][0][m], a1 = vst[ps][1][m], a2 = vst[ps][2][m], a3 = vst[ps][3][m];
-          u32x2 even = {(a0 & 0xffffu) | (a1 << 16), (a2 & 0xffffu) | (a3 << 16)};
-          u32x2 odd = {(a0 >> 16) | (a1 & 0xffff0000u), (a2 >> 16) | (a3 & 0xffff0000u)};
-          *reinterpret_cast<u32x2*>(&vt_lds[(dg * 8 + 2 * m) * VT_STRIDE + pos]) = even;
-          *reinterpret_cast<u32x2*>(&vt_lds[(dg * 8 + 2 * m + 1) * VT_STRIDE + pos]) = odd;
-        }
-      }
-    }
-    __syncthreads();
+    const int64_t off = (int64_t)kv_table[blk] * p.kv_slot_stride +
+                        (int64_t)(k0 - blk * p.block_size) * p.kv_token_stride;
+    KTile::load_async(k_dst, kg + off, k_goff, w);
+    VTile::load_async(v_dst, vg + off, v_goff, w);
+  };
 
+  // one key tile out of a filled stage
+  auto compute = [&](int kt, const uint16_t* k_lds, const uint16_t* v_lds) {
+    const int k0 = kt * BN;
     const bool wave_active = (k0 < w_hi0 && k0 + BN > w_lo0) || (k0 < w_hi1 && k0 + BN > w_lo1);
-    if (!wave_active) continue;
+    if (!wave_active) return;
 
-    // ---- S^T = K Q^T ----------------------------------------------------------
-    f32x16 s_acc[2];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s_acc[nt][i] = 0.0f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(&k_lds[(nt * 32 + c) * K_STRIDE + ks * 16 + h * 8]);
-        s_acc[nt] = mfma_32x32x16<DTYPE>(a, qreg[ks], s_acc[nt]);
-      }
-    }
-
-    // ---- online softmax (log2 domain) -----------------------------------------
+    // ---- S^T = K Q^T -------------------------------------------------------------
+    // The range mask enters as the accumulator's initial value: 0 where the row may
+    // look, -inf where it may not.  A tile inside every row's range of the wave (the
+    // common case) starts from the constant 0; everything after the first product is
+    // the same code for both cases.
     const bool unmasked = (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
-    float mx = -INFINITY;
+    f32x16 s_acc[2];
+    u32x4 ka[2][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      ka[0][ks] = *reinterpret_cast<const u32x4*>(k_lds + k_rd + KTile::at(0, ks * 16));
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      ka[1][ks] = *reinterpret_cast<const u32x4*>(k_lds + k_rd + KTile::at(32, ks * 16));
     if (unmasked) {
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[nt][i]);
-      mx *= p.scale_log2;
+        for (int i = 0; i < 16; ++i) s_acc[nt][i] = 0.0f;
+        s_acc[nt] = mfma_32x32x16<DTYPE>(ka[nt][0], qreg[0], s_acc[nt]);
+      }
     } else {
       const int kb = k0 + 4 * h;
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+      for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int kv = kb + nt * 32 + 8 * (i / 4) + (i % 4);
-          const float s = rng.contains(kv) ? s_acc[nt][i] : -INFINITY;
-          s_acc[nt][i] = s;
-          mx = fmaxf(mx, s);
-        }
-      mx *= p.scale_log2;  // -inf stays -inf (scale > 0)
+        for (int i = 0; i < 16; ++i)
+          s_acc[nt][i] = rng.contains(kb + nt * 32 + 8 * (i / 4) + (i % 4)) ? 0.0f : -INFINITY;
+        s_acc[nt] = mfma_32x32x16<DTYPE>(ka[nt][0], qreg[0], s_acc[nt]);
+      }
     }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int ks = 1; ks < KS; ++ks) s_acc[nt] = mfma_32x32x16<DTYPE>(ka[nt][ks], qreg[ks], s_acc[nt]);
+    // first V^T operands: their latency hides under the softmax arithmetic
+    u32x4 va[2][4];
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) va[0][s2] = VTile::template read_col<true>(v_lds, v_rd, s2 * 16, 0);
+
+    // ---- online softmax (log2 domain) -----------------------------------------
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[nt][i]);
+    mx *= p.scale_log2;  // -inf stays -inf (scale > 0)
     mx = fmaxf(mx, xor32(mx));
     const float m_new = fmaxf(m_run, mx);
     const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
     if (__any(m_new > m_run)) {
-      const float alpha = exp2f(m_run - m_use);  // m_run = -inf -> 0
+      const float alpha = fast_exp2(m_run - m_use);  // m_run = -inf -> 0
       l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
@@ -265,7 +249,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
         for (int i = 0; i < 16; ++i) o_acc[dt][i] *= alpha;
     }
     m_run = m_new;
-
     u32x4 pb[4];
     float lsum = 0.0f;
 #pragma unroll
@@ -275,7 +258,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
         float e[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          e[j] = exp2f(fmaf(s_acc[nt][g * 8 + j], p.scale_log2, -m_use));
+          e[j] = fast_exp2(fmaf(s_acc[nt][g * 8 + j], p.scale_log2, -m_use));
           lsum += e[j];
         }
         u32x4 packed = {pack2<DTYPE>(e[0], e[1]), pack2<DTYPE>(e[2], e[3]), pack2<DTYPE>(e[4], e[5]),
@@ -284,14 +267,31 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
       }
     l_run += lsum;
 
-    // ---- O^T += V^T P^T ---------------------------------------------------------
+    // ---- O^T += V^T P^T: V^T comes out of the row-major V tile by transpose loads -----
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt) {
+      if (dt + 1 < DT) {
 #pragma unroll
-      for (int s2 = 0; s2 < 4; ++s2) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(&vt_lds[(dt * 32 + c) * VT_STRIDE + s2 * 16 + h * 8]);
-        o_acc[dt] = mfma_32x32x16<DTYPE>(a, pb[s2], o_acc[dt]);
+        for (int s2 = 0; s2 < 4; ++s2)
+          va[(dt + 1) & 1][s2] = VTile::template read_col<true>(v_lds, v_rd, s2 * 16, (dt + 1) * 32);
       }
+#pragma unroll
+      for (int s2 = 0; s2 < 4; ++s2) o_acc[dt] = mfma_32x32x16<DTYPE>(va[dt & 1][s2], pb[s2], o_acc[dt]);
+    }
+  };
+
+  // ---- key loop: tile i+1 streams into the other stage while tile i is used ----------
+  if (n_tiles > 0) fetch(runs.tile(0), k_lds0, v_lds0);
+  for (int i = 0; i < n_tiles; i += 2) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
+    if (i + 1 < n_tiles) fetch(runs.tile(i + 1), k_lds1, v_lds1);
+    compute(runs.tile(i), k_lds0, v_lds0);
+    if (i + 1 >= n_tiles) break;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
+    if (i + 2 < n_tiles) fetch(runs.tile(i + 2), k_lds0, v_lds0);
+    compute(runs.tile(i + 1), k_lds1, v_lds1);
   }
 
   // ---- epilogue ------------------------------------------------------------------
