@@ -36,7 +36,9 @@
 //                              tile, B = P rows from LDS
 //   dK^T[dim, key] += Q^T dS   A = Q^T: transpose-load from the Q tile, B = dS
 //
-// Q and dO are staged once, row-major; nothing is stored transposed.  dK/dV of
+// Q and dO tiles go from global memory straight into LDS, row-major; nothing is
+// staged through registers or stored transposed.  The range mask enters S as
+// the accumulator's initial value (0 or -inf).  dK/dV of
 // a key never leave the workgroup's registers until the end, so the
 // per-(row, kv block) private dKV blocks of the plan need no atomics and are
 // written whole (zeros where no query of the row attends).
@@ -158,43 +160,19 @@ __global__ __launch_bounds__(64) void bwd_tile_hull_kernel(const AttnBwdParams p
 // ---------------------------------------------------------------------------
 // main kernel
 // ---------------------------------------------------------------------------
-// 16-byte MFMA operand (8 contraction slots of one row/column) read from an
-// LDS array stored with the CONTRACTION index as its row: element
-// [slot0 + s][col0 + c] for s in [0,8) for the lane's row/column c.  Uses the
-// LDS transpose load: in each group of 16 lanes, lane 4a+b receives element b
-// of the 8-byte chunks addressed by lanes a, a+4, a+8, a+12.
-__device__ __forceinline__ u32x4 lds_read_transposed(const uint16_t* base, int row_stride, int slot0,
-                                                     int col0, int lane) {
-  typedef short s16x4 __attribute__((ext_vector_type(4)));
-  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-  const int j = lane & 15;
-  const int h = lane >> 5;
-  const int cb = col0 + ((lane >> 4) & 1) * 16 + 4 * (j & 3);
-  const uint16_t* p0 = base + (slot0 + 8 * h + (j >> 2)) * row_stride + cb;
-  const uint16_t* p1 = p0 + 4 * row_stride;
-  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
-  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
-  const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-  u32x4 r = {l2[0], l2[1], h2[0], h2[1]};
-  return r;
-}
-
 template <int DTYPE, int D>
 __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
   constexpr int BM = kBwdBM, BN = kBwdBN;
-  constexpr int KS = D / 16;          // k-steps over the head dim
-  constexpr int ROW_STRIDE = D + 8;   // q_lds / do_lds rows (elements)
-  constexpr int T_STRIDE = BM + 8;    // p_lds / ds_lds rows (elements): [key][query]
-  constexpr int CH = D / 8;           // 16-byte chunks per row
-  constexpr int ROWS_PER_PASS = kBwdThreads / CH;
-  constexpr int PASSES = BM / ROWS_PER_PASS;
+  constexpr int KS = D / 16;        // k-steps over the head dim
+  constexpr int T_STRIDE = BM + 8;  // p_lds / ds_lds rows (elements): [key][query]
+  typedef KvTile<D> Tile;           // the Q and dO tiles: 64 queries x D
   // second phase: (32-dim slice, 32-wide tile) units, spread over the 4 waves
   constexpr int SLICES = D / 32;
   constexpr int UPW = SLICES * 2 / 4;  // units per wave: 2 (D=128) or 1 (D=64)
   static_assert(UPW == 1 || UPW == 2, "head dim");
 
-  __shared__ __attribute__((aligned(16))) uint16_t q_lds[BM * ROW_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t do_lds[BM * ROW_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[Tile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t do_lds[Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t p_lds[BN * T_STRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t ds_lds[BN * T_STRIDE];
   __shared__ __attribute__((aligned(16))) int rng_lds[BM * 4];
@@ -230,7 +208,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
   const int q_slot = p.q_block_table[b];
   const int o_slot = p.out_block_table[b];
-  const int n_q_tiles = (seqlen_q + BM - 1) / BM;
+  const int n_q_tiles = (seqlen_q + BM - 1) / BM;  // rows past seqlen_q stay inside the padded block
   const int64_t kv_tile_off = (int64_t)p.kv_block_table[(int64_t)b * p.max_kv_blocks + blk] * p.kv_slot_stride +
                               (int64_t)tok0 * p.kv_token_stride + (int64_t)kv_head * D;
 
@@ -246,6 +224,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       vreg[ks] = *reinterpret_cast<const u32x4*>(vp + ks * 16);
     }
   }
+
   // dK^T / dV^T of (dims of `slice`) x (keys of tile tile0 + u)
   f32x16 dk_acc[UPW], dv_acc[UPW];
 #pragma unroll
@@ -257,7 +236,13 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
 
   const int32_t* hull_row = p.hull + (int64_t)b * p.q_tiles_per_row * 8;
-  const int st_row = tid / CH, st_chunk = tid % CH;
+  // loop-invariant per-lane pieces of the addresses used in the loop
+  uint32_t goff[Tile::LPW];
+  Tile::lane_offsets(goff, q_row_stride, w, lane);
+  const int row_rd = Tile::row_base(c, h) + qi * Tile::ROW32;
+  const int col_rd = Tile::col_base(lane, false) + slice * 32;
+  const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.block_size * q_row_stride;
+  const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.block_size * q_row_stride;
 
   for (int hg = 0; hg < group; ++hg) {
     const int head = kv_head * group + hg;
@@ -268,18 +253,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       if (!active) continue;
       const bool unmasked = (hu[4] <= k0 && k0 + BN <= hu[5]) || (hu[6] <= k0 && k0 + BN <= hu[7]);
 
-      // ---- stage the Q and dO tiles row-major -----------------------------------------
-      u32x4 qst[PASSES], dst[PASSES];
-#pragma unroll
-      for (int ps = 0; ps < PASSES; ++ps) {
-        const int ql = qt * BM + ps * ROWS_PER_PASS + st_row;
-        u32x4 z = {0, 0, 0, 0};
-        const bool ok = ql < seqlen_q;
-        const int64_t qoff = ((int64_t)q_slot * p.block_size + ql) * q_row_stride + (int64_t)head * D + st_chunk * 8;
-        const int64_t ooff = ((int64_t)o_slot * p.block_size + ql) * q_row_stride + (int64_t)head * D + st_chunk * 8;
-        qst[ps] = ok ? *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.q) + qoff) : z;
-        dst[ps] = ok ? *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.dout) + ooff) : z;
-      }
+      // per-row range, lse and delta of the tile's 64 queries
       int4 my_rng = {0, 0, 0, 0};
       float my_lse = INFINITY, my_delta = 0.0f;
       if (tid < BM) {
@@ -297,35 +271,51 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         }
       }
       __syncthreads();  // previous tile fully consumed
-#pragma unroll
-      for (int ps = 0; ps < PASSES; ++ps) {
-        const int r = ps * ROWS_PER_PASS + st_row;
-        *reinterpret_cast<u32x4*>(&q_lds[r * ROW_STRIDE + st_chunk * 8]) = qst[ps];
-        *reinterpret_cast<u32x4*>(&do_lds[r * ROW_STRIDE + st_chunk * 8]) = dst[ps];
+      // ---- Q and dO tiles: global -> LDS directly (rows past seqlen_q are masked below) ----
+      {
+        const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
+        Tile::load_async(q_lds, q_base + off, goff, w);
+        Tile::load_async(do_lds, do_base + off, goff, w);
       }
       if (tid < BM) {
         *reinterpret_cast<int4*>(&rng_lds[tid * 4]) = my_rng;
         lse_lds[tid] = my_lse;
         delta_lds[tid] = my_delta;
       }
+      __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
 
       // ---- phase 1: S = Q K^T, dP = dO V^T on this wave's 32x32 sub-tile ---------------
+      // the range mask enters S as the accumulator's initial value (0 / -inf)
       f32x16 s_acc, dp_acc;
+      const int kv = k0 + ki * 32 + c;
+      if (unmasked) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s_acc[i] = 0.0f;
-        dp_acc[i] = 0.0f;
+        for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int4 rg = *reinterpret_cast<const int4*>(&rng_lds[(qi * 32 + acc_row(i, h)) * 4]);
+          const bool ok = ((unsigned)(kv - rg.x) < (unsigned)rg.y) | ((unsigned)(kv - rg.z) < (unsigned)rg.w);
+          s_acc[i] = ok ? 0.0f : -INFINITY;
+        }
       }
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 aq = *reinterpret_cast<const u32x4*>(&q_lds[(qi * 32 + c) * ROW_STRIDE + ks * 16 + h * 8]);
-        s_acc = mfma_32x32x16<DTYPE>(aq, kreg[ks], s_acc);
-        const u32x4 ad = *reinterpret_cast<const u32x4*>(&do_lds[(qi * 32 + c) * ROW_STRIDE + ks * 16 + h * 8]);
-        dp_acc = mfma_32x32x16<DTYPE>(ad, vreg[ks], dp_acc);
+      for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
+#pragma unroll
+      for (int half = 0; half < KS / 4; ++half) {
+        u32x4 aq[4], ad[4];
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) aq[k4] = Tile::read_row(q_lds, row_rd, 0, half * 4 + k4);
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) ad[k4] = Tile::read_row(do_lds, row_rd, 0, half * 4 + k4);
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) {
+          s_acc = mfma_32x32x16<DTYPE>(aq[k4], kreg[half * 4 + k4], s_acc);
+          dp_acc = mfma_32x32x16<DTYPE>(ad[k4], vreg[half * 4 + k4], dp_acc);
+        }
       }
       // P, dS (lane = key 32ki + c; element i = query 32qi + acc_row(i,h)) -> LDS [key][query]
-      const int kv = k0 + ki * 32 + c;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int qrow = qi * 32 + 8 * g + 4 * h;
@@ -334,16 +324,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         float pv[4], dsv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float e = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));
-          float ds = e * (dp_acc[4 * g + r] - d4[r]);
-          if (!unmasked) {
-            const int4 rg = *reinterpret_cast<const int4*>(&rng_lds[(qrow + r) * 4]);
-            const bool ok = ((unsigned)(kv - rg.x) < (unsigned)rg.y) | ((unsigned)(kv - rg.z) < (unsigned)rg.w);
-            e = ok ? e : 0.0f;
-            ds = ok ? ds : 0.0f;
-          }
-          pv[r] = e;
-          dsv[r] = ds;
+          pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));  // masked: exp2(-inf) = 0
+          dsv[r] = pv[r] * (dp_acc[4 * g + r] - d4[r]);
         }
         u32x2 p4 = {pack2<DTYPE>(pv[0], pv[1]), pack2<DTYPE>(pv[2], pv[3])};
         u32x2 s4 = {pack2<DTYPE>(dsv[0], dsv[1]), pack2<DTYPE>(dsv[2], dsv[3])};
@@ -354,10 +336,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 
       // ---- phase 2: this wave's dim slice ------------------------------------------------
       // dV^T[dim, key] += dO^T[dim, q] P[q, key];  dK^T[dim, key] += Q^T[dim, q] dS[q, key]
+      // (dO^T and Q^T come out of the row-major tiles by transpose loads)
 #pragma unroll
       for (int ks = 0; ks < BM / 16; ++ks) {
-        const u32x4 a_do = lds_read_transposed(do_lds, ROW_STRIDE, ks * 16, slice * 32, lane);
-        const u32x4 a_q = lds_read_transposed(q_lds, ROW_STRIDE, ks * 16, slice * 32, lane);
+        const u32x4 a_do = Tile::template read_col<false>(do_lds, col_rd, ks, 0);
+        const u32x4 a_q = Tile::template read_col<false>(q_lds, col_rd, ks, 0);
 #pragma unroll
         for (int u = 0; u < UPW; ++u) {
           const int row = ((tile0 + u) * 32 + c) * T_STRIDE + ks * 16 + h * 8;
@@ -407,33 +390,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 constexpr int kDqBM = 128;
 constexpr int kDqBN = 64;
 
-// Like lds_read_transposed, but with the contraction slots in accumulator
-// order (slot j of half h = row slot0 + 8*(j/4) + 4h + j%4), so that the other
-// operand can be an accumulator tile.
-__device__ __forceinline__ u32x4 lds_read_transposed_acc_order(const uint16_t* base, int row_stride,
-                                                               int slot0, int col0, int lane) {
-  typedef short s16x4 __attribute__((ext_vector_type(4)));
-  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-  const int j = lane & 15;
-  const int h = lane >> 5;
-  const int cb = col0 + ((lane >> 4) & 1) * 16 + 4 * (j & 3);
-  const uint16_t* p0 = base + (slot0 + 4 * h + (j >> 2)) * row_stride + cb;
-  const uint16_t* p1 = p0 + 8 * row_stride;
-  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
-  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
-  const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-  u32x4 r = {l2[0], l2[1], h2[0], h2[1]};
-  return r;
-}
-
 template <int DTYPE, int D>
 __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnBwdParams p) {
   constexpr int BN = kDqBN;
   constexpr int KS = D / 16;
   constexpr int DT = D / 32;
-  constexpr int K_STRIDE = D + 8;
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[BN * K_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t v_lds[BN * K_STRIDE];
+  typedef KvTile<D> Tile;
+  // two stages of (K tile, V tile); separate arrays so the compiler can tell
+  // the stage being filled from the stage being read
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds0[Tile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds0[Tile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds1[Tile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds1[Tile::SIZE];
   __shared__ int hull_lds[4][4];
 
   const int tid = threadIdx.x;
@@ -514,8 +482,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
     g_lo1 = min(g_lo1, hull_lds[i][2]);
     g_hi1 = max(g_hi1, hull_lds[i][3]);
   }
-  const int kt_begin = min(g_lo0, g_lo1) / BN;
-  const int kt_end = (max(g_hi0, g_hi1) + BN - 1) / BN;
+  const TileRuns runs(g_lo0, g_hi0, g_lo1, g_hi1, BN);
+  const int n_tiles = runs.count();
 
   f32x16 dq_acc[DT];
 #pragma unroll
@@ -526,79 +494,95 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
   const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
-  constexpr int CH = D / 8;
-  constexpr int ROWS_PER_PASS = kBwdThreads / CH;
-  constexpr int PASSES = BN / ROWS_PER_PASS;
-  const int st_row = tid / CH, st_chunk = tid % CH;
+  uint32_t goff[Tile::LPW];
+  Tile::lane_offsets(goff, p.kv_token_stride, w, lane);
+  const int row_rd = Tile::row_base(c, h);
+  const int col_rd = Tile::col_base(lane, true);
 
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
+  auto fetch = [&](int kt, uint16_t* k_dst, uint16_t* v_dst) {
     const int k0 = kt * BN;
-    const bool wg_active = (k0 < g_hi0 && k0 + BN > g_lo0) || (k0 < g_hi1 && k0 + BN > g_lo1);
-    if (!wg_active) continue;
     const int blk = k0 / p.block_size;
-    const int tok0 = k0 - blk * p.block_size;
-    const int64_t tile_off = (int64_t)kv_table[blk] * p.kv_slot_stride + (int64_t)tok0 * p.kv_token_stride;
-    u32x4 kst[PASSES], vst[PASSES];
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      const int64_t off = tile_off + (int64_t)(ps * ROWS_PER_PASS + st_row) * p.kv_token_stride + st_chunk * 8;
-      kst[ps] = *reinterpret_cast<const u32x4*>(kg + off);
-      vst[ps] = *reinterpret_cast<const u32x4*>(vg + off);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-      const int r = ps * ROWS_PER_PASS + st_row;
-      *reinterpret_cast<u32x4*>(&k_lds[r * K_STRIDE + st_chunk * 8]) = kst[ps];
-      *reinterpret_cast<u32x4*>(&v_lds[r * K_STRIDE + st_chunk * 8]) = vst[ps];
-    }
-    __syncthreads();
+    const int64_t off = (int64_t)kv_table[blk] * p.kv_slot_stride +
+                        (int64_t)(k0 - blk * p.block_size) * p.kv_token_stride;
+    Tile::load_async(k_dst, kg + off, goff, w);
+    Tile::load_async(v_dst, vg + off, goff, w);
+  };
 
+  auto compute = [&](int kt, const uint16_t* k_lds, const uint16_t* v_lds) {
+    const int k0 = kt * BN;
     const bool wave_active = (k0 < w_hi0 && k0 + BN > w_lo0) || (k0 < w_hi1 && k0 + BN > w_lo1);
-    if (!wave_active) continue;
+    if (!wave_active) return;
     const bool unmasked = (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
 
     u32x4 dsb[4];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
+      // the range mask enters S^T as the accumulator's initial value (0 / -inf)
       f32x16 s_acc, dp_acc;
+      if (unmasked) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s_acc[i] = 0.0f;
-        dp_acc[i] = 0.0f;
+        for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
+      } else {
+        const int kb = k0 + nt * 32 + 4 * h;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_acc[i] = rng.contains(kb + 8 * (i / 4) + (i % 4)) ? 0.0f : -INFINITY;
       }
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 ak = *reinterpret_cast<const u32x4*>(&k_lds[(nt * 32 + c) * K_STRIDE + ks * 16 + h * 8]);
-        s_acc = mfma_32x32x16<DTYPE>(ak, qreg[ks], s_acc);
-        const u32x4 av = *reinterpret_cast<const u32x4*>(&v_lds[(nt * 32 + c) * K_STRIDE + ks * 16 + h * 8]);
-        dp_acc = mfma_32x32x16<DTYPE>(av, doreg[ks], dp_acc);
+      for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
+      // operands four k-steps at a time; the two accumulation chains interleave
+#pragma unroll
+      for (int half = 0; half < KS / 4; ++half) {
+        u32x4 ka[4], va[4];
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) ka[k4] = Tile::read_row(k_lds, row_rd, nt, half * 4 + k4);
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) va[k4] = Tile::read_row(v_lds, row_rd, nt, half * 4 + k4);
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) {
+          s_acc = mfma_32x32x16<DTYPE>(ka[k4], qreg[half * 4 + k4], s_acc);
+          dp_acc = mfma_32x32x16<DTYPE>(va[k4], doreg[half * 4 + k4], dp_acc);
+        }
       }
-      const int kb = k0 + nt * 32 + 4 * h;
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
         float e[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int i = g * 8 + j;
-          float pr = fast_exp2(fmaf(s_acc[i], p.scale_log2, -lse2));
-          float ds = pr * (dp_acc[i] - delta);
-          if (!unmasked) ds = rng.contains(kb + 8 * (i / 4) + (i % 4)) ? ds : 0.0f;
-          e[j] = ds;
+          const float pr = fast_exp2(fmaf(s_acc[i], p.scale_log2, -lse2));  // masked: exp2(-inf) = 0
+          e[j] = pr * (dp_acc[i] - delta);
         }
         u32x4 packed = {pack2<DTYPE>(e[0], e[1]), pack2<DTYPE>(e[2], e[3]), pack2<DTYPE>(e[4], e[5]),
                         pack2<DTYPE>(e[6], e[7])};
         dsb[nt * 2 + g] = packed;
       }
     }
-    // dQ^T[d, q] += K^T[d, kv] dS^T[kv, q]
+    // dQ^T[d, q] += K^T[d, kv] dS^T[kv, q]: K^T comes out of the K tile by transpose loads
+    u32x4 kt_a[2][4];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int s2 = 0; s2 < 4; ++s2) kt_a[0][s2] = Tile::template read_col<true>(k_lds, col_rd, s2, 0);
 #pragma unroll
-      for (int s2 = 0; s2 < 4; ++s2) {
-        const u32x4 a = lds_read_transposed_acc_order(k_lds, K_STRIDE, s2 * 16, dt * 32, lane);
-        dq_acc[dt] = mfma_32x32x16<DTYPE>(a, dsb[s2], dq_acc[dt]);
+    for (int dt = 0; dt < DT; ++dt) {
+      if (dt + 1 < DT) {
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) kt_a[(dt + 1) & 1][s2] = Tile::template read_col<true>(k_lds, col_rd, s2, dt + 1);
       }
+#pragma unroll
+      for (int s2 = 0; s2 < 4; ++s2) dq_acc[dt] = mfma_32x32x16<DTYPE>(kt_a[dt & 1][s2], dsb[s2], dq_acc[dt]);
+    }
+  };
+
+  if (n_tiles > 0) fetch(runs.tile(0), k_lds0, v_lds0);
+  for (int i = 0; i < n_tiles; i += 2) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
+    if (i + 1 < n_tiles) fetch(runs.tile(i + 1), k_lds1, v_lds1);
+    compute(runs.tile(i), k_lds0, v_lds0);
+    if (i + 1 >= n_tiles) break;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
+    if (i + 2 < n_tiles) fetch(runs.tile(i + 2), k_lds0, v_lds0);
+    compute(runs.tile(i + 1), k_lds1, v_lds1);
   }
 
   if (!q_valid) return;

@@ -76,113 +76,59 @@ __device__ __forceinline__ constexpr int kslot_pos(int r) {
 }
 
 // ---------------------------------------------------------------------------
-// Dense LDS tile [rows][D] of 16-bit elements, filled straight from global
-// memory (no register staging) and read as MFMA operands in both orientations
-// without bank conflicts.
+// LDS tile of 64 rows x D 16-bit elements, filled straight from global memory
+// (global_load_lds, no register staging) and read as an MFMA operand in both
+// orientations, without bank conflicts and with addresses that are a per-lane
+// base plus a compile-time offset (no address arithmetic inside the loops).
 //
-// A row is D/8 16-byte chunks; the chunk at position p of row r holds logical
-// chunk p ^ swz(r).  With swz(r) = (r&3)<<2 | (r>>2)&3 (D = 128; the D = 64
-// variant plays the same game with 128-byte rows):
-//  - 16 lanes reading the same logical chunk of 16 consecutive rows touch 16
-//    different chunk positions (all 64 banks once);
-//  - a transpose load, whose 32 lanes touch 4 consecutive rows x 4 consecutive
-//    chunks, also touches 16 different chunk positions.
 // global_load_lds writes lane l's 16 bytes at (instruction base) + 16*l, so one
-// wave instruction fills 1024 contiguous bytes = 512/D rows, each lane
-// fetching the logical chunk that belongs at its position.
+// wave instruction fills 1024 contiguous bytes: a "group" of G = 512/D rows.
+// All rows of a group share their alignment in the 256-byte bank window (for
+// D = 64 they alternate between its two halves), so rows that are read
+// together must sit in different groups.  Groups are padded by 16 bytes, which
+// puts group g at bank-window offset 16g, and row r of the tile goes to
+//
+//   D = 128:  group 4*(r&3) + (r>>2)&3,   position r>>4 in the group
+//   D =  64:  group 4*(r&1) + (r>>2)&3,   position (r>>1)&1 + 2*(r>>4)
+//
+// so that, within any aligned 16 rows, row r sits at window offset
+// 64*(r&3) + 16*((r>>2)&3) bytes:
+//  - row operand (8 consecutive elements of a row; 16 lanes read 16
+//    consecutive rows at one column): 16 different 16-byte slots;
+//  - column operand (transpose load: one column at 8 rows, the rows being the
+//    contraction index; 32 lanes touch 4 consecutive rows x 64 bytes): four
+//    64-byte windows.
 // ---------------------------------------------------------------------------
 template <int D>
-struct SwzTile {
-  static constexpr int CH = D / 8;                 // chunks per row
-  static constexpr int RPI = 512 / D;              // rows per wave instruction
-  __device__ static __forceinline__ int swz(int r) {
-    return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
-  }
-  // element offset of logical chunk `chunk` of row r
-  __device__ static __forceinline__ int at(int r, int chunk) { return r * D + ((chunk ^ swz(r)) << 3); }
-
-  // Asynchronously copy `rows` rows (multiple of 4*RPI... 64 here) of a global
-  // tile whose rows are `row_stride` elements apart into `tile`; 4 waves.
-  template <int ROWS>
-  __device__ static __forceinline__ void load_async(uint16_t* tile, const uint16_t* g, int64_t row_stride,
-                                                    int wave, int lane) {
-    constexpr int PER_WAVE = ROWS / (4 * RPI);
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; ++i) {
-      const int r0 = (wave * PER_WAVE + i) * RPI;
-      const int r = r0 + lane / CH;
-      const int chunk = (lane % CH) ^ swz(r);
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(g + (int64_t)r * row_stride + chunk * 8),
-          (__attribute__((address_space(3))) void*)(tile + r0 * D), 16, 0, 0);
-    }
-  }
-
-  // MFMA operand of lane (c, h): 8 consecutive elements 16*ks + 8h.. of row `r`.
-  __device__ static __forceinline__ u32x4 read_row(const uint16_t* tile, int r, int ks, int h) {
-    return *reinterpret_cast<const u32x4*>(tile + at(r, 2 * ks + h));
-  }
-
-  // MFMA operand with the tile's ROWS as the contraction index: lane (c, h)
-  // gets column col0 + c at the 8 rows {slot0 + 4h + 0..3, slot0 + 8 + 4h + 0..3}
-  // (accumulator order, ACC_ORDER) or slot0 + 8h + 0..7 (natural order).
-  template <bool ACC_ORDER>
-  __device__ static __forceinline__ u32x4 read_col(const uint16_t* tile, int slot0, int col0, int lane) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    const int j = lane & 15;
-    const int h = lane >> 5;
-    const int d = col0 + ((lane >> 4) & 1) * 16 + 4 * (j & 3);
-    const int r0 = slot0 + (ACC_ORDER ? 4 * h : 8 * h) + (j >> 2);
-    const int r1 = r0 + (ACC_ORDER ? 8 : 4);
-    const uint16_t* p0 = tile + at(r0, d >> 3) + (d & 4);
-    const uint16_t* p1 = tile + at(r1, d >> 3) + (d & 4);
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
-    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-    u32x4 out = {l2[0], l2[1], h2[0], h2[1]};
-    return out;
-  }
-};
-
-// ---------------------------------------------------------------------------
-// LDS tiles of 64 rows x D 16-bit elements whose operand addresses are AFFINE
-// in the loop indices, so every ds_read uses a per-lane base register plus an
-// immediate offset (no address arithmetic inside the key loop).
-//
-// global_load_lds fills 1024 contiguous bytes per wave instruction: a "group"
-// of G = 512/D rows.  Which rows form a group, and the padding between groups,
-// is chosen per access pattern so that the reads are free of bank conflicts:
-//
-//  RowTile  operand = 8 consecutive elements of a row, 16 lanes read 16
-//           consecutive rows (A operand of X K^T-type products).  Row r lives
-//           in group r % NG, so 16 consecutive rows sit in 16 different groups;
-//           groups are 16 bytes apart modulo the 256-byte bank window.
-//  ColTile  operand = one column at 8 rows (transpose load; rows are the
-//           contraction index).  One transpose load touches 4 consecutive rows
-//           x 64 bytes; those rows sit in 4 consecutive groups that are 64
-//           bytes apart modulo the bank window.
-// ---------------------------------------------------------------------------
-template <int D>
-struct RowTile {
+struct KvTile {
   static constexpr int ROWS = 64;
-  static constexpr int G = 512 / D;                // rows per group (4 for D=128, 8 for D=64)
-  static constexpr int NG = ROWS / G;              // groups (16 / 8)
-  static constexpr int GROUP_STRIDE = G * D + 8;   // elements: 1024 B + 16 B
-  static constexpr int SIZE = NG * GROUP_STRIDE;   // elements
-  // element offset of (row r, element e)
-  __device__ static __forceinline__ int at(int r, int e) { return (r % NG) * GROUP_STRIDE + (r / NG) * D + e; }
-  static constexpr int LPW = NG / 4;  // group loads per wave (4 waves fill a tile)
+  static constexpr int G = 512 / D;
+  static constexpr int NG = ROWS / G;
+  static constexpr int GROUP_STRIDE = G * D + 8;  // elements: 1024 B + 16 B
+  static constexpr int SIZE = NG * GROUP_STRIDE;  // elements
+  static constexpr int LPW = NG / 4;              // group loads per wave (4 waves fill a tile)
+  static constexpr int ROW32 = 256;               // element offset of row r + 32 (both head dims)
+  static constexpr int ROW16 = 128;               // element offset of row r + 16
+  static constexpr int ROW8 = 2 * GROUP_STRIDE;   // row r + 8  (r % 16 < 8)
+  static constexpr int ROW4 = GROUP_STRIDE;       // row r + 4  (r % 16 in 0..3 or 8..11)
+
+  __device__ static __forceinline__ int at(int r, int e) {
+    const int grp = D == 128 ? 4 * (r & 3) + ((r >> 2) & 3) : 4 * (r & 1) + ((r >> 2) & 3);
+    const int pos = D == 128 ? (r >> 4) : ((r >> 1) & 1) + 2 * (r >> 4);
+    return grp * GROUP_STRIDE + pos * D + e;
+  }
+  // row held at position `pos` of group `grp`
+  __device__ static __forceinline__ int row_of(int grp, int pos) {
+    return D == 128 ? 16 * pos + 4 * (grp & 3) + (grp >> 2)
+                    : 16 * (pos >> 1) + 4 * (grp & 3) + 2 * (pos & 1) + (grp >> 2);
+  }
   // Byte offsets, from (row 0, the head's first element), of what this lane
   // fetches in each of its wave's group loads.  Loop-invariant.
   __device__ static __forceinline__ void lane_offsets(uint32_t (&off)[LPW], int64_t row_stride, int wave, int lane) {
     constexpr int CH = D / 8;
-    const int sub = lane / CH, chunk = lane % CH;
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const int r = sub * NG + wave * LPW + i;
-      off[i] = (uint32_t)((r * row_stride + chunk * 8) * 2);
-    }
+    for (int i = 0; i < LPW; ++i)
+      off[i] = (uint32_t)((row_of(wave * LPW + i, lane / CH) * row_stride + (lane % CH) * 8) * 2);
   }
   // `g` (wave-uniform) points at (row 0, the head's first element) of the tile.
   __device__ static __forceinline__ void load_async(uint16_t* tile, const uint16_t* g, const uint32_t (&off)[LPW],
@@ -194,62 +140,31 @@ struct RowTile {
                                        (__attribute__((address_space(3))) void*)(tile + (wave * LPW + i) * GROUP_STRIDE),
                                        16, 0, 0);
   }
-};
-
-template <int D>
-struct ColTile {
-  static constexpr int ROWS = 64;
-  static constexpr int G = 512 / D;
-  static constexpr int NG = ROWS / G;
-  static constexpr int GROUP_STRIDE = G * D + 32;  // elements: 1024 B + 64 B
-  static constexpr int SIZE = NG * GROUP_STRIDE;
-  // rows 4m..4m+3 -> 4 consecutive groups, same position inside the group:
-  // group(r) = (r & 3) + 4 * (r / (4 * G)),  sub(r) = (r / 4) % G
-  __device__ static __forceinline__ int at(int r, int e) {
-    return ((r & 3) + 4 * (r / (4 * G))) * GROUP_STRIDE + ((r >> 2) % G) * D + e;
-  }
-  static constexpr int LPW = NG / 4;
-  __device__ static __forceinline__ void lane_offsets(uint32_t (&off)[LPW], int64_t row_stride, int wave, int lane) {
-    constexpr int CH = D / 8;
-    const int sub = lane / CH, chunk = lane % CH;
-#pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const int grp = wave * LPW + i;
-      const int r = (grp >> 2) * (4 * G) + sub * 4 + (grp & 3);
-      off[i] = (uint32_t)((r * row_stride + chunk * 8) * 2);
-    }
-  }
-  __device__ static __forceinline__ void load_async(uint16_t* tile, const uint16_t* g, const uint32_t (&off)[LPW],
-                                                    int wave) {
-    const char* gb = reinterpret_cast<const char*>(g);
-#pragma unroll
-    for (int i = 0; i < LPW; ++i)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gb + off[i]),
-                                       (__attribute__((address_space(3))) void*)(tile + (wave * LPW + i) * GROUP_STRIDE),
-                                       16, 0, 0);
-  }
-  // Per-lane base of the transpose loads: lane (j = lane%16, half-wave h, 16-lane
-  // group q) reads element column 16q + 4(j%4) of row (j/4) + 4h [+ slot offsets].
-  __device__ static __forceinline__ int lane_base(int lane, bool acc_order) {
+  // Row operand of lane (c, h): elements 16*ks + 8h.. of row 32*nt + c at
+  //   tile + row_base(c, h) + nt*ROW32 + ks*16
+  __device__ static __forceinline__ int row_base(int c, int h) { return at(c, 8 * h); }
+  // Column operand of lane l: column 32*ct + (l & 31) at the 8 rows of k-step s2,
+  //   ACC_ORDER: 16*s2 + {4h..4h+3, 8+4h..8+4h+3}   (matches accumulator rows)
+  //   else:      16*s2 + 8h + 0..7
+  // read as two transpose loads at tile + col_base(l) + s2*ROW16 + ct*32 (+ ROW8 or ROW4).
+  __device__ static __forceinline__ int col_base(int lane, bool acc_order) {
     const int j = lane & 15, h = lane >> 5;
-    const int r = (acc_order ? 4 * h : 8 * h) + (j >> 2);
-    return at(r, ((lane >> 4) & 1) * 16 + 4 * (j & 3));
+    return at((acc_order ? 4 * h : 8 * h) + (j >> 2), ((lane >> 4) & 1) * 16 + 4 * (j & 3));
   }
-  // 8 contraction slots starting at row `slot0` (multiple of 16) for column
-  // block `col0` (multiple of 32); `base` from lane_base().  ACC_ORDER: slots
-  // are rows {4h..4h+3, 8+4h..8+4h+3} (accumulator order), else 8h..8h+7.
   template <bool ACC_ORDER>
-  __device__ static __forceinline__ u32x4 read_col(const uint16_t* tile, int base, int slot0, int col0) {
+  __device__ static __forceinline__ u32x4 read_col(const uint16_t* tile, int base, int s2, int ct) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    // rows advance by 16 -> 4 groups (D=128) ; +8 rows (acc order) or +4 rows -> inside-group / next groups
-    const int o0 = at(slot0, col0);
-    const int o1 = ACC_ORDER ? at(slot0 + 8, col0) : at(slot0 + 4, col0);
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + base + o0));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + base + o1));
+    const uint16_t* p0 = tile + base + s2 * ROW16 + ct * 32;
+    const uint16_t* p1 = p0 + (ACC_ORDER ? ROW8 : ROW4);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
     const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
     u32x4 out = {l2[0], l2[1], h2[0], h2[1]};
     return out;
+  }
+  __device__ static __forceinline__ u32x4 read_row(const uint16_t* tile, int base, int nt, int ks) {
+    return *reinterpret_cast<const u32x4*>(tile + base + nt * ROW32 + ks * 16);
   }
 };
 

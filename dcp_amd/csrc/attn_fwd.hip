@@ -67,8 +67,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   constexpr int BN = kFwdBN;
   constexpr int KS = D / 16;  // k-steps of S^T = K Q^T
   constexpr int DT = D / 32;  // 32-row tiles of O^T
-  typedef RowTile<D> KTile;  // read as rows (A operand of S^T)
-  typedef ColTile<D> VTile;  // read as columns (A operand of O^T = V^T P^T)
+  typedef KvTile<D> KTile;  // read as rows (A operand of S^T)
+  typedef KvTile<D> VTile;  // read as columns (A operand of O^T = V^T P^T)
   // two stages of (K tile, V tile); separate arrays so the compiler can tell
   // the stage being filled from the stage being read
   __shared__ __attribute__((aligned(16))) uint16_t k_lds0[KTile::SIZE];
@@ -171,8 +171,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   uint32_t k_goff[KTile::LPW], v_goff[VTile::LPW];
   KTile::lane_offsets(k_goff, p.kv_token_stride, w, lane);
   VTile::lane_offsets(v_goff, p.kv_token_stride, w, lane);
-  const int k_rd = KTile::at(c, 8 * h);         // + nt*32 rows, + ks*16 elements
-  const int v_rd = VTile::lane_base(lane, true);  // + slot / column block offsets
+  const int k_rd = KTile::row_base(c, h);
+  const int v_rd = VTile::col_base(lane, true);
 
   // fill one stage with key tile `kt`
   auto fetch = [&](int kt, uint16_t* k_dst, uint16_t* v_dst) {
@@ -200,10 +200,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
     u32x4 ka[2][KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      ka[0][ks] = *reinterpret_cast<const u32x4*>(k_lds + k_rd + KTile::at(0, ks * 16));
+      ka[0][ks] = KTile::read_row(k_lds, k_rd, 0, ks);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      ka[1][ks] = *reinterpret_cast<const u32x4*>(k_lds + k_rd + KTile::at(32, ks * 16));
+      ka[1][ks] = KTile::read_row(k_lds, k_rd, 1, ks);
     if (unmasked) {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
     // first V^T operands: their latency hides under the softmax arithmetic
     u32x4 va[2][4];
 #pragma unroll
-    for (int s2 = 0; s2 < 4; ++s2) va[0][s2] = VTile::template read_col<true>(v_lds, v_rd, s2 * 16, 0);
+    for (int s2 = 0; s2 < 4; ++s2) va[0][s2] = VTile::template read_col<true>(v_lds, v_rd, s2, 0);
 
     // ---- online softmax (log2 domain) -----------------------------------------
     float mx = -INFINITY;
@@ -273,7 +273,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
       if (dt + 1 < DT) {
 #pragma unroll
         for (int s2 = 0; s2 < 4; ++s2)
-          va[(dt + 1) & 1][s2] = VTile::template read_col<true>(v_lds, v_rd, s2 * 16, (dt + 1) * 32);
+          va[(dt + 1) & 1][s2] = VTile::template read_col<true>(v_lds, v_rd, s2, dt + 1);
       }
 #pragma unroll
       for (int s2 = 0; s2 < 4; ++s2) o_acc[dt] = mfma_32x32x16<DTYPE>(va[dt & 1][s2], pb[s2], o_acc[dt]);
