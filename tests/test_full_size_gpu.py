@@ -1,0 +1,192 @@
+"""BASELINE-size runs on the GPU, checked through size-independent properties
+and seeded samples of the oracle (the full oracle would take hours):
+
+* config 2 (Llama-3-8B shape, 65536 tokens, causal, bs 1024, GQA 32/8):
+  sampled (sequence, head) parity against dense fp64 attention, exact
+  linearity of the backward in dO, bit-reproducibility, HIP-graph replays;
+* config 3 (lambda mask, sink 64 + window 4096) at 32768 tokens: sampled parity;
+* config 5 (262144 x 32 x 128 bf16 block movement): gather -> inverse scatter is
+  the identity bit for bit, padding rows stay untouched, and the 4-way merge is
+  invariant under a permutation of its sources.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import bench
+from oracle import dcp_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(wl, seed=0, graph=False):
+    from dcp_amd.core.instructions import BufferType
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+
+    fw, bw, layout, mask, pairs = bench.build(wl)
+    ex_f, ex_b = bench.make_executors(wl, fw, bw, seed=seed)
+    ex_f.execute(fw, True)
+    ex_b.execute(bw, False)
+    torch.cuda.synchronize()
+    B = BufferType
+    t = {k: ex_f.buffers[k] for k in (B.LOCAL_Q, B.LOCAL_KV, B.LOCAL_OUT, B.LOCAL_LSE)}
+    t.update({k: ex_b.buffers[k] for k in (B.LOCAL_dOUT, B.LOCAL_dQ, B.LOCAL_dKV)})
+    return fw, bw, layout, mask, ex_f, ex_b, t
+
+
+def _sample_check(wl, layout, mask, t, samples):
+    """Dense fp64 attention for a few (sequence, kv head) groups."""
+    from dcp_amd.core.instructions import BufferType as B
+
+    hb = wl["head_block"]
+    group = wl["n_heads"] // wl["n_groups"]
+    seq_off = np.concatenate(([0], np.cumsum(wl["seqlens"])))
+    total = int(seq_off[-1])
+    worst = dict(out=0.0, lse=0.0, dq=0.0, dkv=0.0)
+    for s, kvh in samples:
+        L = wl["seqlens"][s]
+        # LOCAL order is (head block, sequence, block): a sequence is contiguous inside a head block
+        hblk = kvh * group // hb  # first q head block of this kv head's group
+        n_hblk = max(1, group // hb)
+        sl_kv = slice(kvh * total + int(seq_off[s]), kvh * total + int(seq_off[s]) + L)
+        kv = t[B.LOCAL_KV][sl_kv].float().cpu().numpy()  # [L, 2, 1, D]
+        qs, douts, outs, lses, dqs = [], [], [], [], []
+        for j in range(n_hblk):
+            sl = slice((hblk + j) * total + int(seq_off[s]), (hblk + j) * total + int(seq_off[s]) + L)
+            qs.append(t[B.LOCAL_Q][sl].float().cpu().numpy())
+            douts.append(t[B.LOCAL_dOUT][sl].float().cpu().numpy())
+            outs.append(t[B.LOCAL_OUT][sl].float().cpu().numpy())
+            lses.append(t[B.LOCAL_LSE][:, sl].cpu().numpy())
+            dqs.append(t[B.LOCAL_dQ][sl].float().cpu().numpy())
+        q, dout = np.concatenate(qs, axis=1), np.concatenate(douts, axis=1)
+        m = mask[int(seq_off[s]) : int(seq_off[s]) + L].numpy()
+        r_out, r_lse, r_dq, r_dkv = oracle.dense_reference(q, kv, m, [L], dout=dout, dtype=np.float64)
+        rel = lambda g, r: float((np.abs(g - r) / np.maximum(1.0, np.abs(r))).max())
+        worst["out"] = max(worst["out"], rel(np.concatenate(outs, axis=1), r_out))
+        worst["lse"] = max(worst["lse"], float(np.abs(np.concatenate(lses, axis=0) - r_lse).max()))
+        worst["dq"] = max(worst["dq"], rel(np.concatenate(dqs, axis=1), r_dq))
+        worst["dkv"] = max(worst["dkv"], rel(t[B.LOCAL_dKV][sl_kv].float().cpu().numpy(), r_dkv))
+    return worst
+
+
+def test_config2_llama_shape_sampled_parity_linearity_determinism(gpu):
+    from dcp_amd.core.instructions import BufferType as B
+
+    wl = bench.workload("llama3_8b_causal_64k")
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl)
+    order = np.argsort(wl["seqlens"])
+    samples = [(int(order[0]), 0), (int(order[len(order) // 2]), 5), (int(order[3]), 7)]  # short and medium sequences
+    worst = _sample_check(wl, layout, mask, t, samples)
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+    assert bool(torch.isfinite(t[B.LOCAL_LSE]).all()) and bool(torch.isfinite(t[B.LOCAL_dKV].float()).all())
+
+    # bit-reproducible: no atomics anywhere on the path
+    dq0, dkv0, out0 = t[B.LOCAL_dQ].clone(), t[B.LOCAL_dKV].clone(), t[B.LOCAL_OUT].clone()
+    ex_f.execute(fw, True)
+    ex_b.execute(bw, False)
+    torch.cuda.synchronize()
+    assert torch.equal(t[B.LOCAL_OUT], out0) and torch.equal(t[B.LOCAL_dQ], dq0) and torch.equal(t[B.LOCAL_dKV], dkv0)
+
+    # the backward is linear in dO, and scaling by 2 commutes with every rounding
+    t[B.LOCAL_dOUT].mul_(2)
+    ex_b.execute(bw, False)
+    torch.cuda.synchronize()
+    assert torch.equal(t[B.LOCAL_dQ], dq0 * 2) and torch.equal(t[B.LOCAL_dKV], dkv0 * 2)
+
+
+def test_config2_hip_graph_replays_match_eager(gpu):
+    from dcp_amd.core.instructions import BufferType as B
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+
+    wl = bench.workload("smoke")
+    fw, bw, layout, mask, pairs = bench.build(wl)
+    ex = get_executor(wl["head_block"], wl["head_dim"], None, fw_exec_plan=fw, bw_exec_plan=bw, use_cudagraph=True)
+    ex.prepare(forward=True)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q = torch.randn(ex.buffers[B.LOCAL_Q].shape, generator=g, device="cuda").to(torch.bfloat16)
+    kv = torch.randn(ex.buffers[B.LOCAL_KV].shape, generator=g, device="cuda").to(torch.bfloat16)
+    eager_out, eager_lse = ex.forward(q, kv)
+    ex.capture_cudagraph()
+    assert ex.cuda_graph is not None
+    for i in range(3):  # replays with eager work and synchronisation in between
+        ex.buffers[B.LOCAL_OUT].zero_()
+        ex.buffers[B.BUFFER_OUT].fill_(float(i))
+        torch.cuda.synchronize()
+        out, lse = ex.forward(q, kv)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager_out) and torch.equal(lse, eager_lse), i
+    # new inputs through the same graph
+    q2 = q * 0.5
+    out2, _ = ex.forward(q2, kv)
+    ex.cuda_graph = None
+    ref2, _ = ex.forward(q2, kv)
+    assert torch.equal(out2, ref2)
+
+
+def test_config3_lambda_mask_sampled_parity(gpu):
+    wl = bench.workload("lambda_128k")
+    wl = dict(wl, seqlens=bench.lognormal_lengths(32768, 8192, 256, 16384, seed=1))
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl, seed=2)
+    order = np.argsort(wl["seqlens"])
+    samples = [(int(order[-1]) if wl["seqlens"][order[-1]] <= 9000 else int(order[len(order) // 2]), 3)]
+    worst = _sample_check(wl, layout, mask, t, samples)
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+
+
+def test_config5_block_movement_full_size(gpu):
+    from dcp_amd.ops.fused_ops import flash_attn_update_out_lse, fused_copy_bf16_varlen
+
+    tokens, heads, d, bs = 262144, 32, 128, 512
+    n_blocks = tokens // bs
+    numel = bs * heads * d
+    rng = np.random.default_rng(0)
+    perm = rng.permutation(n_blocks)
+    n_tok = rng.integers(1, bs + 1, n_blocks)  # ragged blocks: only the first n tokens move
+    n_tok[:8] = bs
+    g = torch.Generator(device="cuda").manual_seed(0)
+    src = torch.randn(tokens, heads, d, device="cuda", generator=g).to(torch.bfloat16)
+    packed = torch.full_like(src, 7.0)
+    back = torch.zeros_like(src)
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    i32 = lambda v: torch.tensor(np.ascontiguousarray(v), dtype=torch.int32, device="cuda")
+    ident, stride = np.arange(n_blocks), i32([numel] * n_blocks)
+    n_el = i32(n_tok * heads * d)
+    fused_copy_bf16_varlen(i64([src.data_ptr()] * n_blocks), i32(ident), stride, i64([packed.data_ptr()] * n_blocks),
+                           i32(perm), stride, n_el, numel, 128)
+    fused_copy_bf16_varlen(i64([packed.data_ptr()] * n_blocks), i32(perm), stride, i64([back.data_ptr()] * n_blocks),
+                           i32(ident), stride, n_el, numel, 128)
+    torch.cuda.synchronize()
+    valid = (torch.arange(bs, device="cuda")[None, :] < torch.tensor(n_tok, device="cuda")[:, None]).reshape(-1)
+    s3, b3, p3 = (x.view(torch.int16).reshape(tokens, -1) for x in (src, back, packed))
+    assert torch.equal(b3[valid], s3[valid])  # gather then inverse scatter: identity, bit for bit
+    assert bool((b3[~valid] == 0).all())  # rows past n_tokens are never written
+    inv = np.argsort(perm)
+    pad_rows = ~valid.reshape(n_blocks, bs)[torch.tensor(inv, device="cuda")].reshape(-1)
+    seven = torch.tensor(7.0, dtype=torch.bfloat16).view(torch.int16).item()
+    assert bool((p3[pad_rows] == seven).all())
+    del packed, back
+
+    # merge: permuting the sources of every op leaves the result unchanged up to rounding
+    n_src = 4
+    blocks = n_blocks  # all 262144 tokens: 4 x 2 GiB of partial outputs
+    outs = torch.randn(n_src * blocks, bs, heads, d, device="cuda", generator=g).to(torch.bfloat16)
+    lses = torch.rand(heads, n_src * blocks, bs, device="cuda", generator=g) * 10 - 5
+    table = rng.permutation(n_src * blocks).reshape(blocks, n_src)
+    results = []
+    for order in ([0, 1, 2, 3], [2, 0, 3, 1]):
+        dst_out = torch.empty(blocks * bs, heads, d, device="cuda", dtype=torch.bfloat16)
+        dst_lse = torch.empty(heads, blocks * bs, device="cuda")
+        flash_attn_update_out_lse(outs, dst_out, lses, dst_lse, heads, i32(table[:, order]), i32(np.arange(blocks) * bs),
+                                  i32([bs] * blocks), i32([n_src] * blocks), bs, numel, heads * d, bs, 1,
+                                  n_src * blocks * bs, blocks * bs, d, n_src, 64)
+        results.append((dst_out, dst_lse))
+    torch.cuda.synchronize()
+    assert float((results[0][1] - results[1][1]).abs().max()) <= 1e-5
+    a, b = results[0][0].float(), results[1][0].float()
+    assert float(((a - b).abs() / a.abs().clamp(min=1.0)).max()) <= 2e-2  # one bf16 ulp of summation order
+    # and a sampled block against the oracle
+    b0 = 17
+    o, l = oracle.merge_out_lse(outs[table[b0]].float().cpu().numpy(), lses[:, table[b0]].permute(1, 0, 2).cpu().numpy())
+    assert np.abs(results[0][0][b0 * bs : (b0 + 1) * bs].float().cpu().numpy() - o).max() <= 2e-2
+    assert np.abs(results[0][1][:, b0 * bs : (b0 + 1) * bs].cpu().numpy() - l).max() <= 1e-3
