@@ -80,51 +80,70 @@ __global__ __launch_bounds__(256) void merge_out_lse_kernel(
   const int n_src = block_lengths[op];
   const int32_t* table = src_block_table + (int64_t)op * max_n_blocks_per_op;
   const float* lse_row = src_lse + h * src_lse_head_stride + t * lse_token_stride;
-
-  float m = -INFINITY;
-  for (int j = 0; j < n_src; ++j) {
-    const float l = lse_row[table[j] * lse_block_stride];
-    if (lse_is_finite(l)) m = fmaxf(m, l);
-  }
-  float new_lse = -1.0f;
-  if (m != -INFINITY) {
-    float s = 0.0f;
-    for (int j = 0; j < n_src; ++j) {
-      const float l = lse_row[table[j] * lse_block_stride];
-      if (lse_is_finite(l)) s += expf(l - m);
-    }
-    new_lse = m + logf(s);
-  }
-
+  const raw* out_row = src_out + t * out_token_stride + (int64_t)h * head_dim;
   const int64_t dst_tok = (int64_t)dst_token_offsets[op] + t;
   const int n_words = head_dim / VN;
+
+  // One pass over the sources, four at a time: the four LSEs and the four
+  // 16-byte words are requested before any arithmetic, then folded into a
+  // running (max, sum, weighted out) triple.
+  float row_lse = -1.0f;  // the same in every iteration: it only depends on the LSEs
   for (int w = g; w < n_words; w += lanes_per_row) {
+    float m = -INFINITY, ssum = 0.0f;
     float acc[VN];
 #pragma unroll
     for (int i = 0; i < VN; ++i) acc[i] = 0.0f;
-    if (m != -INFINITY) {
-      for (int j = 0; j < n_src; ++j) {
-        const int b = table[j];
-        const float l = lse_row[b * lse_block_stride];
-        if (!lse_is_finite(l)) continue;
-        const float wgt = expf(l - new_lse);
-        const raw* p = src_out + b * out_block_stride + t * out_token_stride +
-                       (int64_t)h * head_dim + (int64_t)w * VN;
-        if constexpr (VECTOR) {
-          fma_vec16<DTYPE>(acc, wgt, *reinterpret_cast<const u32x4*>(p));
-        } else {
-          acc[0] += wgt * Elem<DTYPE>::load(*p);
-        }
+    for (int j0 = 0; j0 < n_src; j0 += 4) {
+      float l[4];
+      u32x4 x[4];
+      raw x1[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = min(j0 + u, n_src - 1);  // tail: re-read the last source, ignored below
+        const int64_t blk = table[j];
+        l[u] = lse_row[blk * lse_block_stride];
+        const raw* p = out_row + blk * out_block_stride + (int64_t)w * VN;
+        if constexpr (VECTOR) x[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        else x1[u] = *p;
       }
+      float m_new = m;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (j0 + u >= n_src || !lse_is_finite(l[u])) l[u] = -INFINITY;
+        m_new = fmaxf(m_new, l[u]);
+      }
+      if (m_new == -INFINITY) continue;  // nothing finite so far
+      const float rescale = expf(m - m_new);  // m = -inf -> 0
+      ssum *= rescale;
+#pragma unroll
+      for (int i = 0; i < VN; ++i) acc[i] *= rescale;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float wgt = expf(l[u] - m_new);  // ignored source: exp(-inf) = 0, but its data may be
+        if (l[u] == -INFINITY) continue;       // anything, so it is skipped, not multiplied by 0
+        ssum += wgt;
+        if constexpr (VECTOR) fma_vec16<DTYPE>(acc, wgt, x[u]);
+        else acc[0] += wgt * Elem<DTYPE>::load(x1[u]);
+      }
+      m = m_new;
+    }
+    float new_lse = -1.0f;
+    if (m != -INFINITY) {
+      new_lse = m + logf(ssum);
+      const float inv = 1.0f / ssum;
+#pragma unroll
+      for (int i = 0; i < VN; ++i) acc[i] *= inv;
     }
     raw* q = dst_out + dst_tok * out_token_stride + (int64_t)h * head_dim + (int64_t)w * VN;
     if constexpr (VECTOR) {
-      *reinterpret_cast<u32x4*>(q) = pack_vec16<DTYPE>(acc);
+      __builtin_nontemporal_store(pack_vec16<DTYPE>(acc), reinterpret_cast<u32x4*>(q));
     } else {
       *q = Elem<DTYPE>::store(acc[0]);
     }
+    row_lse = new_lse;
   }
-  if (g == 0) dst_lse[h * dst_lse_head_stride + dst_tok * lse_token_stride] = new_lse;
+  // after every read of the sources' LSEs (the destination may be one of them)
+  if (g == 0) dst_lse[h * dst_lse_head_stride + dst_tok * lse_token_stride] = row_lse;
 }
 
 template <int DTYPE>
