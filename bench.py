@@ -149,7 +149,7 @@ def kernel_times(ex_f, ex_b, fw, bw, steps):
     return {name: dict(launches=n, avg_ms=total / n, ms_per_step=total / steps) for name, (n, total) in rep.items()}
 
 
-def movement_microbench(iters=5):
+def movement_microbench(iters=5, bs=512):
     """BASELINE config 5: 262144 tokens x 32 heads x 128, bf16, 512-token
     blocks; gather through a seeded block permutation, inverse scatter, then a
     4-way (out, lse) merge.  Returns GB/s from events on the launch stream."""
@@ -157,7 +157,7 @@ def movement_microbench(iters=5):
     from dcp_amd import _lib
     from dcp_amd.ops.fused_ops import flash_attn_update_out_lse, fused_copy_bf16_varlen
 
-    tokens, heads, d, bs = 262144, 32, 128, 512
+    tokens, heads, d = 262144, 32, 128
     n_blocks = tokens // bs
     numel = bs * heads * d
     rng = np.random.default_rng(0)

@@ -81,6 +81,10 @@ struct AttnBwdParams {
   int64_t dkv_slot_stride;
   int64_t dkv_token_stride;
   int n_out_slots;
+  int dkv_xcd_group;     // dK/dV work items sharing one Q/dO stream (the key tiles of a row)
+  int dq_xcd_group;      // dQ work items sharing one K/V stream
+  int64_t n_dkv_items;   // batch * n_heads_kv * kv_tiles_per_row
+  int64_t n_dq_items;    // batch * n_heads_q * dq_tiles_per_row
   int q_tiles_per_row;   // ceil(block_size / 64): query tiles of the dK/dV kernel
   int dq_tiles_per_row;  // ceil(block_size / 128): query tiles of the dQ kernel
   int kv_tiles_per_row;  // max_kv_blocks * block_size / 64
@@ -191,7 +195,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const int tile0 = UPW == 2 ? 0 : (w & 1);
 
   // ---- which (row, kv head, key tile) ------------------------------------------
-  int wg = blockIdx.x;
+  // the key tiles of a row share its Q/dO tiles: keep them on one XCD
+  int wg = xcd_logical_id(blockIdx.x, p.dkv_xcd_group, p.n_dkv_items);
+  if (wg < 0) return;
   const int kt = wg % p.kv_tiles_per_row;
   wg /= p.kv_tiles_per_row;
   const int kv_head = wg % p.n_heads_kv;
@@ -410,7 +416,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   const int c = lane & 31;
   const int h = lane >> 5;
 
-  int wg = blockIdx.x;
+  // the query tiles and grouped heads of a row share its K/V: keep them on one XCD
+  int wg = xcd_logical_id(blockIdx.x, p.dq_xcd_group, p.n_dq_items);
+  if (wg < 0) return;
   const int qt = wg % p.dq_tiles_per_row;
   wg /= p.dq_tiles_per_row;
   const int head = wg % p.n_heads_q;
@@ -604,8 +612,8 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.block_size * p.n_heads_q;
   const int64_t chunks = (rows + ROWS - 1) / ROWS;
   DCP_REQUIRE(chunks <= 65535, "attn_bwd: block of %lld (token, head) rows is too large", (long long)rows);
-  const int64_t n_dkv = (int64_t)p.batch * p.n_heads_kv * p.kv_tiles_per_row;
-  const int64_t n_dq = (int64_t)p.batch * p.n_heads_q * p.dq_tiles_per_row;
+  const int64_t n_dkv = xcd_grid_size(p.n_dkv_items, p.dkv_xcd_group);
+  const int64_t n_dq = xcd_grid_size(p.n_dq_items, p.dq_xcd_group);
   DCP_REQUIRE(n_dkv < ((int64_t)1 << 31) && n_dq < ((int64_t)1 << 31), "attn_bwd: grid too large");
   {
     KernelTimer timer("bwd_prep_kernel", stream);
@@ -719,6 +727,10 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
   p.q_tiles_per_row = (block_size + kBwdBM - 1) / kBwdBM;
   p.dq_tiles_per_row = (block_size + kDqBM - 1) / kDqBM;
   p.kv_tiles_per_row = max_kv_blocks * (block_size / kBwdBN);
+  p.n_dkv_items = (int64_t)batch * n_heads_kv * p.kv_tiles_per_row;
+  p.n_dq_items = (int64_t)batch * n_heads_q * p.dq_tiles_per_row;
+  p.dkv_xcd_group = p.kv_tiles_per_row;
+  p.dq_xcd_group = p.dq_tiles_per_row * (n_heads_q / n_heads_kv);
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * kLog2e;
   if (dtype == DCP_DTYPE_BF16)

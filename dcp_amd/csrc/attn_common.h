@@ -168,6 +168,32 @@ struct KvTile {
   }
 };
 
+// ---------------------------------------------------------------------------
+// XCD-aware workgroup numbering.  The 256 CUs sit in 8 XCDs, each with its own
+// L2, and consecutive workgroup ids are dealt round-robin to the XCDs.  Work
+// items that stream the same tiles from HBM (the query tiles and grouped heads
+// of one row share its K/V; the key tiles of one row share its Q/dO) should
+// therefore NOT have consecutive ids: with `group` such items per shared
+// stream, hardware id w is mapped to the logical item
+//
+//   ((w / (8*group)) * 8 + w % 8) * group + (w % (8*group)) / 8
+//
+// so that the `group` items of one stream all have the same w % 8 (one XCD, one
+// copy in one L2) while neighbouring streams still spread over all 8 XCDs.
+// The grid is rounded up to a multiple of 8*group; ids past `total` are idle.
+// ---------------------------------------------------------------------------
+constexpr int kNumXcd = 8;
+__device__ __forceinline__ int xcd_logical_id(int w, int group, int64_t total) {
+  const int per_super = kNumXcd * group;
+  const int super = w / per_super, r = w - super * per_super;
+  const int64_t id = ((int64_t)super * kNumXcd + (r % kNumXcd)) * group + r / kNumXcd;
+  return id < total ? (int)id : -1;
+}
+inline int64_t xcd_grid_size(int64_t total, int group) {
+  const int64_t per_super = (int64_t)kNumXcd * group;
+  return (total + per_super - 1) / per_super * per_super;
+}
+
 // The (at most two) runs of key tiles a workgroup has to visit, from the hull
 // of its rows' ranges.  Tiles are BN keys wide.
 struct TileRuns {

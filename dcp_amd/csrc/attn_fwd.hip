@@ -55,6 +55,8 @@ struct AttnFwdParams {
   int64_t kv_token_stride;
   int n_out_slots;
   int q_tiles_per_row;
+  int xcd_group;     // work items per shared K/V stream
+  int64_t n_items;   // batch * n_heads_q * q_tiles_per_row
   float scale_log2;  // softmax_scale * log2(e)
 };
 
@@ -84,7 +86,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   const int h = lane >> 5;
 
   // ---- which (row, head, q tile) ----------------------------------------
-  int wg = blockIdx.x;
+  // the query tiles and grouped heads of a row share its K/V: keep them on one XCD
+  int wg = xcd_logical_id(blockIdx.x, p.xcd_group, p.n_items);
+  if (wg < 0) return;
   const int qt = wg % p.q_tiles_per_row;
   wg /= p.q_tiles_per_row;
   const int head = wg % p.n_heads_q;
@@ -373,7 +377,9 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   p.n_out_slots = n_out_slots;
   p.q_tiles_per_row = (block_size + kFwdBM - 1) / kFwdBM;
   p.scale_log2 = softmax_scale * kLog2e;
-  const int64_t n_wg = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
+  p.n_items = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
+  p.xcd_group = p.q_tiles_per_row * (n_heads_q / n_heads_kv);
+  const int64_t n_wg = xcd_grid_size(p.n_items, p.xcd_group);
   DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_fwd: grid too large");
   dim3 grid((unsigned)n_wg), block(kFwdThreads);
   KernelTimer timer("attn_fwd_kernel", stream);

@@ -58,8 +58,10 @@ __device__ __forceinline__ bool lse_is_finite(float l) {
 // the destination may alias a source of the same op.
 // grid: (ops, row chunks)
 // ---------------------------------------------------------------------------
+constexpr int kMergeThreads = 256;
+
 template <int DTYPE, bool VECTOR>
-__global__ __launch_bounds__(256) void merge_out_lse_kernel(
+__global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
     const typename Elem<DTYPE>::raw* src_out, typename Elem<DTYPE>::raw* dst_out,
     const float* src_lse, float* dst_lse, int n_head, const int32_t* __restrict__ src_block_table,
     const int32_t* __restrict__ dst_token_offsets, const int32_t* __restrict__ n_tokens_per_block,
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(256) void merge_out_lse_kernel(
   constexpr int VN = VECTOR ? Vec16<DTYPE>::N : 1;
   const int op = blockIdx.x;
   const int n_tok = n_tokens_per_block[op];
-  const int rows_per_wg = 256 / lanes_per_row;
+  const int rows_per_wg = kMergeThreads / lanes_per_row;
   const int row = blockIdx.y * rows_per_wg + threadIdx.x / lanes_per_row;
   const int g = threadIdx.x % lanes_per_row;
   const int t = row / n_head;
@@ -164,7 +166,7 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
   const int n_words = vec ? head_dim / VN : head_dim;
   int lpr = 1;
   while (lpr < 64 && n_words % (lpr * 2) == 0) lpr *= 2;
-  const int rows_per_wg = 256 / lpr;
+  const int rows_per_wg = kMergeThreads / lpr;
   const int64_t rows = (int64_t)block_size * n_head;
   const int64_t row_chunks = (rows + rows_per_wg - 1) / rows_per_wg;
   DCP_REQUIRE(row_chunks <= 65535, "merge: block of %lld (token, head) rows is too large",
@@ -172,7 +174,7 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
   dim3 grid(n_red_ops, (unsigned)row_chunks);
   KernelTimer timer("merge_out_lse_kernel", stream);
   auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, (hipStream_t)stream, (const raw*)src_out,
+    hipLaunchKernelGGL(kernel, grid, dim3(kMergeThreads), 0, (hipStream_t)stream, (const raw*)src_out,
                        (raw*)dst_out, src_lse, dst_lse, n_head, src_block_table,
                        dst_token_offsets, n_tokens_per_block, block_lengths, out_block_stride,
                        out_token_stride, lse_block_stride, lse_token_stride, src_lse_head_stride,
