@@ -29,6 +29,15 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per launch of the backward kernel pair, from rocprofv3 --pmc runs of this
+# script (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the counter
+# reads for the 2 GiB -> 2 GiB copy kernel of the same run: x2.0 and x1.0).  Counters
+# cannot be read from inside the benchmark, so the figure is per workload and is only
+# reported for the workload it was measured on.
+MEASURED_TRAFFIC_BYTES = {
+    "llama3_8b_causal_64k": int(((1409263.8 + 1856554.1) * 2.0 + (1302542.9 + 581640.1) * 1.0) * 1024),
+}
+
 
 # ---------------------------------------------------------------------------
 # workloads (BASELINE.json configs)
@@ -314,7 +323,8 @@ def main():
     fwd_tflops = flops_fwd / (fwd["avg_ms"] * 1e-3) / 1e12
     roofline = dict(
         bound="mfma", kernel="attn_bwd_dkv_kernel+attn_bwd_dq_kernel", achieved=round(bwd_tflops, 2),
-        peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4), traffic=None,
+        peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4),
+        traffic=MEASURED_TRAFFIC_BYTES.get(args.workload),
         flops_per_launch=2.5 * flops_fwd, avg_launch_ms=round(bwd_ms, 4),
     )
     extra = dict(
