@@ -280,8 +280,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       // ---- Q and dO tiles: global -> LDS directly (rows past seqlen_q are masked below) ----
       {
         const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
-        Tile::load_async(q_lds, q_base + off, goff, w);
-        Tile::load_async(do_lds, do_base + off, goff, w);
+        Tile::load_async(lds_address(q_lds), q_base + off, goff, w);
+        Tile::load_async(lds_address(do_lds), do_base + off, goff, w);
       }
       if (tid < BM) {
         *reinterpret_cast<int4*>(&rng_lds[tid * 4]) = my_rng;
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   const int row_rd = Tile::row_base(c, h);
   const int col_rd = Tile::col_base(lane, true);
 
-  auto fetch = [&](int kt, uint16_t* k_dst, uint16_t* v_dst) {
+  auto fetch = [&](int kt, uint32_t k_dst, uint32_t v_dst) {
     const int k0 = kt * BN;
     const int blk = k0 / p.block_size;
     const int64_t off = (int64_t)kv_table[blk] * p.kv_slot_stride +
@@ -580,16 +580,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
     }
   };
 
-  if (n_tiles > 0) fetch(runs.tile(0), k_lds0, v_lds0);
+  const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
+  const uint32_t v_at0 = lds_address(v_lds0), v_at1 = lds_address(v_lds1);
+  if (n_tiles > 0) fetch(runs.tile(0), k_at0, v_at0);
   for (int i = 0; i < n_tiles; i += 2) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
-    if (i + 1 < n_tiles) fetch(runs.tile(i + 1), k_lds1, v_lds1);
+    if (i + 1 < n_tiles) fetch(runs.tile(i + 1), k_at1, v_at1);
     compute(runs.tile(i), k_lds0, v_lds0);
     if (i + 1 >= n_tiles) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
-    if (i + 2 < n_tiles) fetch(runs.tile(i + 2), k_lds0, v_lds0);
+    if (i + 2 < n_tiles) fetch(runs.tile(i + 2), k_at0, v_at0);
     compute(runs.tile(i + 1), k_lds1, v_lds1);
   }
 

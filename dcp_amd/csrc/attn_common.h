@@ -51,12 +51,12 @@ __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
 __device__ __forceinline__ int wave_min(int x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x = min(x, __shfl_xor(x, o));
-  return x;
+  return __builtin_amdgcn_readfirstlane(x);  // the same in every lane: let the compiler know
 }
 __device__ __forceinline__ int wave_max(int x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x = max(x, __shfl_xor(x, o));
-  return x;
+  return __builtin_amdgcn_readfirstlane(x);
 }
 
 // Row index (within a 32-row MFMA tile) of accumulator element i for a lane
@@ -76,7 +76,7 @@ __device__ __forceinline__ constexpr int kslot_pos(int r) {
 }
 
 // ---------------------------------------------------------------------------
-// LDS tile of 64 rows x D 16-bit elements, filled straight from global memory
+// LDS tile of 64 rows x D 16-bit elements, filled by NW waves straight from global memory
 // (global_load_lds, no register staging) and read as an MFMA operand in both
 // orientations, without bank conflicts and with addresses that are a per-lane
 // base plus a compile-time offset (no address arithmetic inside the loops).
@@ -99,14 +99,20 @@ __device__ __forceinline__ constexpr int kslot_pos(int r) {
 //    contraction index; 32 lanes touch 4 consecutive rows x 64 bytes): four
 //    64-byte windows.
 // ---------------------------------------------------------------------------
-template <int D>
+// LDS byte address of a __shared__ object
+template <typename T>
+__device__ __forceinline__ uint32_t lds_address(T* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)p;
+}
+
+template <int D, int NW = 4>
 struct KvTile {
   static constexpr int ROWS = 64;
   static constexpr int G = 512 / D;
   static constexpr int NG = ROWS / G;
   static constexpr int GROUP_STRIDE = G * D + 8;  // elements: 1024 B + 16 B
   static constexpr int SIZE = NG * GROUP_STRIDE;  // elements
-  static constexpr int LPW = NG / 4;              // group loads per wave (4 waves fill a tile)
+  static constexpr int LPW = NG / NW;             // group loads per wave (NW waves fill a tile)
   static constexpr int ROW32 = 256;               // element offset of row r + 32 (both head dims)
   static constexpr int ROW16 = 128;               // element offset of row r + 16
   static constexpr int ROW8 = 2 * GROUP_STRIDE;   // row r + 8  (r % 16 < 8)
@@ -131,14 +137,27 @@ struct KvTile {
       off[i] = (uint32_t)((row_of(wave * LPW + i, lane / CH) * row_stride + (lane % CH) * 8) * 2);
   }
   // `g` (wave-uniform) points at (row 0, the head's first element) of the tile.
-  __device__ static __forceinline__ void load_async(uint16_t* tile, const uint16_t* g, const uint32_t (&off)[LPW],
+  //
+  // The load is written as assembly on purpose.  Through the builtin the compiler sees
+  // an instruction that touches both global memory and LDS, and as long as one is in
+  // flight it turns every LDS wait of the wave into a wait for ALL outstanding LDS
+  // reads (lgkmcnt(0)), which serialises operand prefetch with the MFMAs for the whole
+  // time a tile is streaming in, i.e. always.  Here the compiler tracks nothing, so the
+  // kernels must (and do) order these loads themselves: s_waitcnt vmcnt(0) and a
+  // workgroup barrier between a load and the first read of its stage, a barrier between
+  // the last read of a stage and the load that refills it.
+  // `tile_at` is the tile's LDS byte address (lds_address() of the array).
+  __device__ static __forceinline__ void load_async(uint32_t tile_at, const uint16_t* g, const uint32_t (&off)[LPW],
                                                     int wave) {
     const char* gb = reinterpret_cast<const char*>(g);
 #pragma unroll
-    for (int i = 0; i < LPW; ++i)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gb + off[i]),
-                                       (__attribute__((address_space(3))) void*)(tile + (wave * LPW + i) * GROUP_STRIDE),
-                                       16, 0, 0);
+    for (int i = 0; i < LPW; ++i) {
+      const uint32_t lds_at = __builtin_amdgcn_readfirstlane(tile_at + (wave * LPW + i) * GROUP_STRIDE * 2);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :
+                   : "s"(lds_at), "v"(gb + off[i])
+                   : "memory");
+    }
   }
   // Row operand of lane (c, h): elements 16*ks + 8h.. of row 32*nt + c at
   //   tile + row_base(c, h) + nt*ROW32 + ks*16
@@ -194,6 +213,19 @@ inline int64_t xcd_grid_size(int64_t total, int group) {
   return (total + per_super - 1) / per_super * per_super;
 }
 
+// Workgroup barrier between the phases of a kernel whose LDS tiles are filled
+// by global_load_lds.  It waits for this wave's LDS accesses (lgkmcnt) but, unlike
+// __syncthreads(), not for its outstanding global loads, so tiles requested a phase
+// or two ahead stay in flight; wait_loads() is the explicit vmcnt(0) a wave issues
+// before the barrier that publishes the tiles it requested.  The "memory" clobber
+// keeps the compiler from moving memory accesses across the barrier.
+__device__ __forceinline__ void phase_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+// s_waitcnt vmcnt(0), expcnt and lgkmcnt fields at their maximum: as a builtin, so that
+// the compiler's own wait-count bookkeeping knows the tile loads have landed
+__device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // The (at most two) runs of key tiles a workgroup has to visit, from the hull
 // of its rows' ranges.  Tiles are BN keys wide.
 struct TileRuns {
@@ -212,6 +244,56 @@ struct TileRuns {
   }
   __device__ __forceinline__ int count() const { return (b0 - a0) + (b1 - a1); }
   __device__ __forceinline__ int tile(int i) const { return i < b0 - a0 ? a0 + i : a1 + (i - (b0 - a0)); }
+};
+
+// A row's kv block table in LDS, and a cursor that walks the key tiles of a
+// TileRuns list and yields each tile's element offset in the paged K/V buffer.
+// A table lookup straight from global memory is a dependent load the wave has to
+// sit out (a microsecond) before it can even request the tile; done once per tile
+// it costs more than the tile's arithmetic.  The cursor touches the table only
+// when it enters a new block, and then in LDS.
+constexpr int kSlotTableCap = 1024;  // blocks of a row held in LDS; rows with more read the rest from global memory
+
+__device__ __forceinline__ void load_slot_table(int* slot_lds, const int32_t* kv_table, int max_kv_blocks, int tid,
+                                                int n_threads) {
+  for (int i = tid; i < min(max_kv_blocks, kSlotTableCap); i += n_threads) slot_lds[i] = kv_table[i];
+}
+
+struct TileCursor {
+  int index;    // position in the tile list
+  int tile;     // key tile number (BN keys each)
+  int pos;      // tile within its block
+  int blk;      // block within the row
+  int64_t off;  // element offset of the tile's first key row
+
+  __device__ __forceinline__ static int slot(const int* slot_lds, const int32_t* kv_table, int blk) {
+    return blk < kSlotTableCap ? slot_lds[blk] : kv_table[blk];
+  }
+  __device__ __forceinline__ void seek(const TileRuns& runs, int i, int tiles_per_block, const int* slot_lds,
+                                       const int32_t* kv_table, int64_t slot_stride, int64_t tile_stride) {
+    index = i;
+    tile = runs.tile(i);
+    blk = tile / tiles_per_block;
+    pos = tile - blk * tiles_per_block;
+    off = (int64_t)slot(slot_lds, kv_table, blk) * slot_stride + pos * tile_stride;
+  }
+  // to the next tile of the list (call only while index + 1 < runs.count())
+  __device__ __forceinline__ void advance(const TileRuns& runs, int tiles_per_block, const int* slot_lds,
+                                          const int32_t* kv_table, int64_t slot_stride, int64_t tile_stride) {
+    if (index + 1 == runs.b0 - runs.a0) {  // jump to the second run
+      seek(runs, index + 1, tiles_per_block, slot_lds, kv_table, slot_stride, tile_stride);
+      return;
+    }
+    ++index;
+    ++tile;
+    ++pos;
+    off += tile_stride;
+    if (pos == tiles_per_block) {
+      pos = 0;
+      ++blk;
+      off = (int64_t)slot(slot_lds, kv_table, blk) * slot_stride;
+    }
+  }
 };
 
 struct RangePair {

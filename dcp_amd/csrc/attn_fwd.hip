@@ -14,6 +14,12 @@
 // rescale factor is a per-lane scalar, and the masked range of the row lives
 // in four registers.
 //
+// Software pipeline inside a wave: S^T of tile j+1 is multiplied while tile j is
+// exponentiated, MFMA by MFMA in one instruction stream, so the matrix pipe and the
+// vector ALU work at the same time instead of taking turns; O^T += V^T P^T of tile
+// j follows as a dense run of MFMAs that the other wave of the SIMD can fill with
+// its own arithmetic.
+//
 // K and V tiles go from global memory straight into LDS (global_load_lds, no
 // register staging), in two stages: the next tile streams in while the current
 // one is multiplied.  The row order and padding of each tile are chosen so that
@@ -78,6 +84,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   __shared__ __attribute__((aligned(16))) uint16_t k_lds1[KTile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds1[VTile::SIZE];
   __shared__ int hull_lds[4][4];
+  __shared__ int slot_lds[kSlotTableCap];
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -140,6 +147,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   const int core_hi0 = wave_min(rng.len0 > 0 ? rng.s0 + rng.len0 : 0);
   const int core_lo1 = wave_max(rng.len1 > 0 ? rng.s1 : big);
   const int core_hi1 = wave_min(rng.len1 > 0 ? rng.s1 + rng.len1 : 0);
+  const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
+  load_slot_table(slot_lds, kv_table, p.max_kv_blocks, tid, kFwdThreads);
   if (lane == 0) {
     hull_lds[w][0] = w_lo0;
     hull_lds[w][1] = w_hi0;
@@ -169,7 +178,6 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
 
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
-  const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
 
   // loop-invariant per-lane pieces of every address used in the key loop
   uint32_t k_goff[KTile::LPW], v_goff[VTile::LPW];
@@ -178,124 +186,198 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   const int k_rd = KTile::row_base(c, h);
   const int v_rd = VTile::col_base(lane, true);
 
-  // fill one stage with key tile `kt`
-  auto fetch = [&](int kt, uint16_t* k_dst, uint16_t* v_dst) {
-    const int k0 = kt * BN;
-    const int blk = k0 / p.block_size;
-    const int64_t off = (int64_t)kv_table[blk] * p.kv_slot_stride +
-                        (int64_t)(k0 - blk * p.block_size) * p.kv_token_stride;
-    KTile::load_async(k_dst, kg + off, k_goff, w);
-    VTile::load_async(v_dst, vg + off, v_goff, w);
+  // The cursor runs two tiles ahead of the tile being exponentiated: it names the K
+  // tile to request next.  V of a tile is requested one iteration after its K, from the
+  // offset remembered then.
+  const int tiles_per_block = p.block_size / BN;
+  const int64_t tile_stride = (int64_t)BN * p.kv_token_stride;
+  TileCursor cursor;
+  auto cursor_next = [&]() {
+    if (cursor.index + 1 < n_tiles) cursor.advance(runs, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
+    else ++cursor.index;  // past the end: nothing left to request
+  };
+  const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
+  const uint32_t v_at0 = lds_address(v_lds0), v_at1 = lds_address(v_lds1);
+  // does any row of this wave see key tile `tile` / does every row see all of it
+  auto wave_sees = [&](int tile) -> bool {
+    const int k0 = tile * BN;
+    return (k0 < w_hi0 && k0 + BN > w_lo0) || (k0 < w_hi1 && k0 + BN > w_lo1);
+  };
+  auto wave_sees_all = [&](int tile) -> bool {
+    const int k0 = tile * BN;
+    return (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
   };
 
-  // one key tile out of a filled stage
-  auto compute = [&](int kt, const uint16_t* k_lds, const uint16_t* v_lds) {
-    const int k0 = kt * BN;
-    const bool wave_active = (k0 < w_hi0 && k0 + BN > w_lo0) || (k0 < w_hi1 && k0 + BN > w_lo1);
-    if (!wave_active) return;
+  // MFMA i of S^T = K Q^T: key half i & 1, k-step i >> 1 (the two halves alternate so
+  // that consecutive MFMAs are independent)
+  auto k_operand = [&](const uint16_t* k_lds, int i) { return KTile::read_row(k_lds, k_rd, i & 1, i >> 1); };
 
-    // ---- S^T = K Q^T -------------------------------------------------------------
-    // The range mask enters as the accumulator's initial value: 0 where the row may
-    // look, -inf where it may not.  A tile inside every row's range of the wave (the
-    // common case) starts from the constant 0; everything after the first product is
-    // the same code for both cases.
-    const bool unmasked = (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
-    f32x16 s_acc[2];
-    u32x4 ka[2][KS];
+  // S^T of tile i on its own.  The range mask enters as the accumulator's initial
+  // value: 0 where the row may look, -inf where it may not.
+  auto multiply_qk = [&](int tile, const uint16_t* k_lds, f32x16 (&s_out)[2]) {
+    if (wave_sees_all(tile)) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      ka[0][ks] = KTile::read_row(k_lds, k_rd, 0, ks);
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      ka[1][ks] = KTile::read_row(k_lds, k_rd, 1, ks);
-    if (unmasked) {
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_acc[nt][i] = 0.0f;
-        s_acc[nt] = mfma_32x32x16<DTYPE>(ka[nt][0], qreg[0], s_acc[nt]);
-      }
+        for (int e = 0; e < 16; ++e) s_out[nt][e] = 0.0f;
     } else {
-      const int kb = k0 + 4 * h;
+      const int kb = tile * BN + 4 * h;
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-          s_acc[nt][i] = rng.contains(kb + nt * 32 + 8 * (i / 4) + (i % 4)) ? 0.0f : -INFINITY;
-        s_acc[nt] = mfma_32x32x16<DTYPE>(ka[nt][0], qreg[0], s_acc[nt]);
-      }
+        for (int e = 0; e < 16; ++e)
+          s_out[nt][e] = rng.contains(kb + nt * 32 + 8 * (e / 4) + (e % 4)) ? 0.0f : -INFINITY;
     }
+    constexpr int N = 2 * KS, AHEAD = 3;
+    u32x4 ka[4];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int i2 = 0; i2 < AHEAD; ++i2) ka[i2] = k_operand(k_lds, i2);
 #pragma unroll
-      for (int ks = 1; ks < KS; ++ks) s_acc[nt] = mfma_32x32x16<DTYPE>(ka[nt][ks], qreg[ks], s_acc[nt]);
-    // first V^T operands: their latency hides under the softmax arithmetic
-    u32x4 va[2][4];
-#pragma unroll
-    for (int s2 = 0; s2 < 4; ++s2) va[0][s2] = VTile::template read_col<true>(v_lds, v_rd, s2, 0);
+    for (int i2 = 0; i2 < N; ++i2) {
+      if (i2 + AHEAD < N) ka[(i2 + AHEAD) & 3] = k_operand(k_lds, i2 + AHEAD);
+      s_out[i2 & 1] = mfma_32x32x16<DTYPE>(ka[i2 & 3], qreg[i2 >> 1], s_out[i2 & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from being hoisted into more registers
+    }
+  };
 
-    // ---- online softmax (log2 domain) -----------------------------------------
+  // ---- online softmax (log2 domain), in pieces so that it can be interleaved ----
+  u32x4 pb[4];          // P^T of the current tile, packed: the B operand of O^T += V^T P^T
+  float alpha = 1.0f;   // pending rescale of O^T (applied before the tile's P^T is multiplied in)
+  bool rescale = false;
+  float m_use = 0.0f, lsum = 0.0f;
+  auto softmax_max = [&](const f32x16 (&sc)[2]) {
     float mx = -INFINITY;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[nt][i]);
+      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[nt][e]);
     mx *= p.scale_log2;  // -inf stays -inf (scale > 0)
     mx = fmaxf(mx, xor32(mx));
     const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-    if (__any(m_new > m_run)) {
-      const float alpha = fast_exp2(m_run - m_use);  // m_run = -inf -> 0
-      l_run *= alpha;
+    m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+    rescale = __any(m_new > m_run);
+    alpha = fast_exp2(m_run - m_use);  // m_run = -inf -> 0; 1 where the max did not move
+    l_run *= alpha;
+    m_run = m_new;
+    lsum = 0.0f;
+  };
+  // elements 2c, 2c+1 of the 32 this lane holds
+  auto softmax_pair = [&](const f32x16 (&sc)[2], int c2) {
+    const int nt = c2 >> 3, e = (c2 & 7) * 2;
+    const float e0 = fast_exp2(fmaf(sc[nt][e], p.scale_log2, -m_use));
+    const float e1 = fast_exp2(fmaf(sc[nt][e + 1], p.scale_log2, -m_use));
+    lsum += e0 + e1;
+    pb[nt * 2 + (e >> 3)][(e & 7) >> 1] = pack2<DTYPE>(e0, e1);
+  };
+  auto apply_rescale = [&]() {
+    if (rescale) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[dt][i] *= alpha;
+        for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
     }
-    m_run = m_new;
-    u32x4 pb[4];
-    float lsum = 0.0f;
+  };
+  auto softmax = [&](const f32x16 (&sc)[2]) {
+    softmax_max(sc);
+#pragma unroll
+    for (int c2 = 0; c2 < 16; ++c2) softmax_pair(sc, c2);
+    l_run += lsum;
+  };
+
+  // S^T of the next tile and the softmax of the current one in one instruction stream:
+  // every MFMA is followed by its share of the softmax arithmetic, so that the matrix
+  // pipe and the vector ALU of the SIMD are busy at the same time.  Operands are read
+  // three MFMAs ahead.
+  auto multiply_qk_with_softmax = [&](const uint16_t* k_lds, f32x16 (&s_out)[2], const f32x16 (&sc)[2]) {
+    constexpr int N = 2 * KS;     // MFMAs
+    constexpr int AHEAD = 3;
+    constexpr int FIRST = N >= 8 ? 3 : 1;  // MFMAs that carry the max; the pairs follow
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        float e[8];
+      for (int e = 0; e < 16; ++e) s_out[nt][e] = 0.0f;
+    u32x4 ka[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          e[j] = fast_exp2(fmaf(s_acc[nt][g * 8 + j], p.scale_log2, -m_use));
-          lsum += e[j];
-        }
-        u32x4 packed = {pack2<DTYPE>(e[0], e[1]), pack2<DTYPE>(e[2], e[3]), pack2<DTYPE>(e[4], e[5]),
-                        pack2<DTYPE>(e[6], e[7])};
-        pb[nt * 2 + g] = packed;
+    for (int i = 0; i < AHEAD; ++i) ka[i] = k_operand(k_lds, i);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (i + AHEAD < N) ka[(i + AHEAD) & 3] = k_operand(k_lds, i + AHEAD);
+      s_out[i & 1] = mfma_32x32x16<DTYPE>(ka[i & 3], qreg[i >> 1], s_out[i & 1]);
+      if (i == 0) softmax_max(sc);
+      if (i >= FIRST) {
+        const int lo = (i - FIRST) * 16 / (N - FIRST), hi = (i + 1 - FIRST) * 16 / (N - FIRST);
+#pragma unroll
+        for (int c2 = lo; c2 < hi; ++c2) softmax_pair(sc, c2);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     l_run += lsum;
+  };
 
-    // ---- O^T += V^T P^T: V^T comes out of the row-major V tile by transpose loads -----
+  // O^T += V^T P^T: V^T comes out of the row-major V tile by transpose loads, read
+  // two MFMAs ahead; consecutive MFMAs go to different 32-row tiles of O^T
+  auto multiply_pv = [&](const uint16_t* v_lds) {
+    constexpr int N = 4 * DT;
+    constexpr int AHEAD = 2;
+    auto v_operand = [&](int i) { return VTile::template read_col<true>(v_lds, v_rd, i / DT, i % DT); };
+    u32x4 va[4];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      if (dt + 1 < DT) {
+    for (int i = 0; i < AHEAD; ++i) va[i] = v_operand(i);
 #pragma unroll
-        for (int s2 = 0; s2 < 4; ++s2)
-          va[(dt + 1) & 1][s2] = VTile::template read_col<true>(v_lds, v_rd, s2, dt + 1);
-      }
-#pragma unroll
-      for (int s2 = 0; s2 < 4; ++s2) o_acc[dt] = mfma_32x32x16<DTYPE>(va[dt & 1][s2], pb[s2], o_acc[dt]);
+    for (int i = 0; i < N; ++i) {
+      if (i + AHEAD < N) va[(i + AHEAD) & 3] = v_operand(i + AHEAD);
+      o_acc[i % DT] = mfma_32x32x16<DTYPE>(va[i & 3], pb[i / DT], o_acc[i % DT]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // ---- key loop: tile i+1 streams into the other stage while tile i is used ----------
-  if (n_tiles > 0) fetch(runs.tile(0), k_lds0, v_lds0);
-  for (int i = 0; i < n_tiles; i += 2) {
+  // ---- key loop --------------------------------------------------------------------
+  // Iteration j multiplies S^T of tile j+1 while it exponentiates tile j, then adds
+  // tile j to O^T.  K tile j+1 and V tile j are in LDS by then; K tile j+2 and V tile
+  // j+1 stream into the stages that K tile j and V tile j-1 have left.
+  f32x16 s_a[2], s_b[2];
+  int tile_cur = 0, tile_nxt = 0;  // key tile numbers of list entries j and j+1
+  int64_t v_off = 0;               // offset of list entry j+1 (its V is requested in iteration j)
+  auto iteration = [&](int j, f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2], const uint16_t* k_nxt, uint32_t k_fill,
+                       const uint16_t* v_cur, uint32_t v_fill) {
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
-    if (i + 1 < n_tiles) fetch(runs.tile(i + 1), k_lds1, v_lds1);
-    compute(runs.tile(i), k_lds0, v_lds0);
-    if (i + 1 >= n_tiles) break;
+    __syncthreads();  // K tile j+1 and V tile j are filled; nobody reads K tile j or V tile j-1 any more
+    if (j + 2 < n_tiles) KTile::load_async(k_fill, kg + cursor.off, k_goff, w);
+    if (j + 1 < n_tiles) VTile::load_async(v_fill, vg + v_off, v_goff, w);
+    const bool cur = wave_sees(tile_cur), nxt = j + 1 < n_tiles && wave_sees(tile_nxt);
+    if (cur && nxt && wave_sees_all(tile_nxt)) {
+      multiply_qk_with_softmax(k_nxt, s_nxt, s_cur);
+    } else {
+      if (nxt) multiply_qk(tile_nxt, k_nxt, s_nxt);
+      if (cur) softmax(s_cur);
+    }
+    if (cur) {
+      apply_rescale();
+      multiply_pv(v_cur);
+    }
+    tile_cur = tile_nxt;
+    tile_nxt = cursor.tile;
+    v_off = cursor.off;
+    cursor_next();
+  };
+  if (n_tiles > 0) {
+    cursor.seek(runs, 0, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
+    tile_cur = cursor.tile;
+    KTile::load_async(k_at0, kg + cursor.off, k_goff, w);
+    VTile::load_async(v_at0, vg + cursor.off, v_goff, w);
+    cursor_next();
+    tile_nxt = cursor.tile;
+    v_off = cursor.off;
+    if (n_tiles > 1) KTile::load_async(k_at1, kg + cursor.off, k_goff, w);
+    cursor_next();
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
-    if (i + 2 < n_tiles) fetch(runs.tile(i + 2), k_lds0, v_lds0);
-    compute(runs.tile(i + 1), k_lds1, v_lds1);
+    __syncthreads();
+    if (wave_sees(tile_cur)) multiply_qk(tile_cur, k_lds0, s_a);
+    for (int j = 0; j < n_tiles; j += 2) {
+      iteration(j, s_a, s_b, k_lds1, k_at0, v_lds0, v_at1);
+      if (j + 1 >= n_tiles) break;
+      iteration(j + 1, s_b, s_a, k_lds0, k_at1, v_lds1, v_at0);
+    }
   }
 
   // ---- epilogue ------------------------------------------------------------------

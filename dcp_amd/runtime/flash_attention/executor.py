@@ -23,6 +23,7 @@ from __future__ import annotations
 from collections import defaultdict
 from typing import Dict, List, Optional, Tuple
 
+import math
 import numpy as np
 import torch
 
@@ -314,7 +315,8 @@ def _handle_memcpy(exec: AttentionExecutor, instr: MemcpyInstr):
     for (dtype, block_numel), args in args_cache["lse"].items():
         if dtype != torch.float32:
             raise ValueError(f"Unsupported dtype {dtype}")
-        fused_copy_fp32_varlen_lse(*args, block_numel, 128)
+        # the tile argument only has to divide the block (the reference fixes 128, :808)
+        fused_copy_fp32_varlen_lse(*args, block_numel, math.gcd(block_numel, 128))
     torch.cuda.nvtx.range_pop()
 
 
