@@ -56,7 +56,7 @@ __device__ __forceinline__ bool lse_is_finite(float l) {
 // transaction), so no cross-lane traffic is needed.  Because the group sits
 // inside one wave and each lane only overwrites elements it has already read,
 // the destination may alias a source of the same op.
-// grid: (ops, row chunks)
+// grid: (ops, token chunks x heads)
 // ---------------------------------------------------------------------------
 constexpr int kMergeThreads = 256;
 
@@ -72,11 +72,13 @@ __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
   constexpr int VN = VECTOR ? Vec16<DTYPE>::N : 1;
   const int op = blockIdx.x;
   const int n_tok = n_tokens_per_block[op];
+  // A workgroup takes consecutive tokens of ONE head: its LSE reads and its LSE store are
+  // then contiguous floats ([head][token] layout) instead of one 4-byte access per cache
+  // line, and every token's head_dim elements are still one contiguous piece.
   const int rows_per_wg = kMergeThreads / lanes_per_row;
-  const int row = blockIdx.y * rows_per_wg + threadIdx.x / lanes_per_row;
+  const int h = blockIdx.y % n_head;
+  const int t = (blockIdx.y / n_head) * rows_per_wg + threadIdx.x / lanes_per_row;
   const int g = threadIdx.x % lanes_per_row;
-  const int t = row / n_head;
-  const int h = row - t * n_head;
   if (t >= n_tok) return;
 
   const int n_src = block_lengths[op];
@@ -167,10 +169,9 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
   int lpr = 1;
   while (lpr < 64 && n_words % (lpr * 2) == 0) lpr *= 2;
   const int rows_per_wg = kMergeThreads / lpr;
-  const int64_t rows = (int64_t)block_size * n_head;
-  const int64_t row_chunks = (rows + rows_per_wg - 1) / rows_per_wg;
+  const int64_t row_chunks = (int64_t)((block_size + rows_per_wg - 1) / rows_per_wg) * n_head;
   DCP_REQUIRE(row_chunks <= 65535, "merge: block of %lld (token, head) rows is too large",
-              (long long)rows);
+              (long long)block_size * n_head);
   dim3 grid(n_red_ops, (unsigned)row_chunks);
   KernelTimer timer("merge_out_lse_kernel", stream);
   auto launch = [&](auto kernel) {
