@@ -409,6 +409,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   __shared__ __attribute__((aligned(16))) uint16_t k_lds1[Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds1[Tile::SIZE];
   __shared__ int hull_lds[4][4];
+  __shared__ int slot_lds[kSlotTableCap];
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -475,6 +476,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   const int core_hi0 = wave_min(rng.len0 > 0 ? rng.s0 + rng.len0 : 0);
   const int core_lo1 = wave_max(rng.len1 > 0 ? rng.s1 : big);
   const int core_hi1 = wave_min(rng.len1 > 0 ? rng.s1 + rng.len1 : 0);
+  const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
+  load_slot_table(slot_lds, kv_table, p.max_kv_blocks, tid, kBwdThreads);
   if (lane == 0) {
     hull_lds[w][0] = w_lo0;
     hull_lds[w][1] = w_hi0;
@@ -501,19 +504,20 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
 
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
-  const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
   uint32_t goff[Tile::LPW];
   Tile::lane_offsets(goff, p.kv_token_stride, w, lane);
   const int row_rd = Tile::row_base(c, h);
   const int col_rd = Tile::col_base(lane, true);
 
-  auto fetch = [&](int kt, uint32_t k_dst, uint32_t v_dst) {
-    const int k0 = kt * BN;
-    const int blk = k0 / p.block_size;
-    const int64_t off = (int64_t)kv_table[blk] * p.kv_slot_stride +
-                        (int64_t)(k0 - blk * p.block_size) * p.kv_token_stride;
-    Tile::load_async(k_dst, kg + off, goff, w);
-    Tile::load_async(v_dst, vg + off, goff, w);
+  // the cursor names the tile to request next (one ahead of the tile being multiplied)
+  const int tiles_per_block = p.block_size / BN;
+  const int64_t tile_stride = (int64_t)BN * p.kv_token_stride;
+  TileCursor cursor;
+  auto fetch = [&](uint32_t k_dst, uint32_t v_dst) {
+    Tile::load_async(k_dst, kg + cursor.off, goff, w);
+    Tile::load_async(v_dst, vg + cursor.off, goff, w);
+    if (cursor.index + 1 < n_tiles)
+      cursor.advance(runs, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
   };
 
   auto compute = [&](int kt, const uint16_t* k_lds, const uint16_t* v_lds) {
@@ -582,16 +586,19 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
 
   const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
   const uint32_t v_at0 = lds_address(v_lds0), v_at1 = lds_address(v_lds1);
-  if (n_tiles > 0) fetch(runs.tile(0), k_at0, v_at0);
+  if (n_tiles > 0) {
+    cursor.seek(runs, 0, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
+    fetch(k_at0, v_at0);
+  }
   for (int i = 0; i < n_tiles; i += 2) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
-    if (i + 1 < n_tiles) fetch(runs.tile(i + 1), k_at1, v_at1);
+    if (i + 1 < n_tiles) fetch(k_at1, v_at1);
     compute(runs.tile(i), k_lds0, v_lds0);
     if (i + 1 >= n_tiles) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
-    if (i + 2 < n_tiles) fetch(runs.tile(i + 2), k_at0, v_at0);
+    if (i + 2 < n_tiles) fetch(k_at0, v_at0);
     compute(runs.tile(i + 1), k_lds1, v_lds1);
   }
 
