@@ -29,12 +29,15 @@
 //                                                 per register group
 //   P, dS -> LDS as [key][query] with 8-byte stores
 //
-// Phase 2: each wave owns a 32-wide slice of the head dim and contracts over
-// the whole tile:
+// Phase 2: each wave owns one of the two products for one half of the head dim
+// and all 64 keys, and contracts over the tile's 64 queries:
 //
 //   dV^T[dim, key] += dO^T P   A = dO^T: transpose-load from the row-major dO
 //                              tile, B = P rows from LDS
 //   dK^T[dim, key] += Q^T dS   A = Q^T: transpose-load from the Q tile, B = dS
+//
+// so that every operand read from LDS feeds two MFMAs (a 2x2 block of
+// accumulators per k-step).
 //
 // Q and dO tiles go from global memory straight into LDS, row-major; nothing is
 // staged through registers or stored transposed.  The range mask enters S as
@@ -170,18 +173,20 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   constexpr int KS = D / 16;        // k-steps over the head dim
   constexpr int T_STRIDE = BM + 8;  // p_lds / ds_lds rows (elements): [key][query]
   typedef KvTile<D> Tile;           // the Q and dO tiles: 64 queries x D
-  // second phase: (32-dim slice, 32-wide tile) units, spread over the 4 waves
-  constexpr int SLICES = D / 32;
-  constexpr int UPW = SLICES * 2 / 4;  // units per wave: 2 (D=128) or 1 (D=64)
-  static_assert(UPW == 1 || UPW == 2, "head dim");
+  // second phase: a wave owns one of the two products (dV^T or dK^T) for one half of the
+  // head dim and all 64 keys: DB x 2 accumulator blocks that share DB + 2 operand reads
+  // per k-step
+  constexpr int DB = D / 64;  // 32-dim blocks per wave: 2 (D=128) or 1 (D=64)
 
   __shared__ __attribute__((aligned(16))) uint16_t q_lds[Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t do_lds[Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t p_lds[BN * T_STRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t ds_lds[BN * T_STRIDE];
-  __shared__ __attribute__((aligned(16))) int rng_lds[BM * 4];
-  __shared__ __attribute__((aligned(16))) float lse_lds[BM];
-  __shared__ __attribute__((aligned(16))) float delta_lds[BM];
+  // two stages of the per-query scalars: the next step's are fetched during this step
+  __shared__ __attribute__((aligned(16))) int rng_lds[2][BM * 4];
+  __shared__ __attribute__((aligned(16))) float lse_lds[2][BM];
+  __shared__ __attribute__((aligned(16))) float delta_lds[2][BM];
+  __shared__ unsigned long long mask_lds[2];
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -190,9 +195,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const int h = lane >> 5;
   const int qi = w >> 1;  // query sub-tile of this wave in phase 1
   const int ki = w & 1;   // key sub-tile of this wave in phase 1
-  // phase 2: this wave's dim slice; with UPW == 2 it covers both 32-wide tiles
-  const int slice = UPW == 2 ? w : (w >> 1);
-  const int tile0 = UPW == 2 ? 0 : (w & 1);
+  const bool is_dk = (w & 1) != 0;  // phase 2: this wave accumulates dK^T (else dV^T) ...
+  const int dhalf = w >> 1;         // ... for dims [dhalf * D/2, (dhalf + 1) * D/2)
 
   // ---- which (row, kv head, key tile) ------------------------------------------
   // the key tiles of a row share its Q/dO tiles: keep them on one XCD
@@ -231,66 +235,111 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
   }
 
-  // dK^T / dV^T of (dims of `slice`) x (keys of tile tile0 + u)
-  f32x16 dk_acc[UPW], dv_acc[UPW];
+  // dK^T or dV^T of (dim block db of this wave's half) x (key tile u)
+  f32x16 acc[DB][2];
 #pragma unroll
-  for (int u = 0; u < UPW; ++u)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      dk_acc[u][i] = 0.0f;
-      dv_acc[u][i] = 0.0f;
-    }
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[db][u][i] = 0.0f;
 
   const int32_t* hull_row = p.hull + (int64_t)b * p.q_tiles_per_row * 8;
   // loop-invariant per-lane pieces of the addresses used in the loop
   uint32_t goff[Tile::LPW];
   Tile::lane_offsets(goff, q_row_stride, w, lane);
   const int row_rd = Tile::row_base(c, h) + qi * Tile::ROW32;
-  const int col_rd = Tile::col_base(lane, false) + slice * 32;
+  const int col_rd = Tile::col_base(lane, false) + dhalf * (D / 2);
   const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.block_size * q_row_stride;
   const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.block_size * q_row_stride;
 
-  for (int hg = 0; hg < group; ++hg) {
-    const int head = kv_head * group + hg;
-    for (int qt = 0; qt < n_q_tiles; ++qt) {
-      const int32_t* hu = hull_row + qt * 8;
-      const int lo0 = hu[0], hi0 = hu[1], lo1 = hu[2], hi1 = hu[3];
-      const bool active = (k0 < hi0 && k0 + BN > lo0) || (k0 < hi1 && k0 + BN > lo1);
-      if (!active) continue;
-      const bool unmasked = (hu[4] <= k0 && k0 + BN <= hu[5]) || (hu[6] <= k0 && k0 + BN <= hu[7]);
+  // ---- which 64-query tiles of the row see these keys (the same for every head) ----------
+  // bit qt of `act`: some row of tile qt sees some key of the tile; of `unm`: every row sees
+  // every key.  Taken once from the per-tile hulls, so the loop never waits for a table.
+  {
+    bool a = false, u = false;
+    if (tid < 64 && tid < n_q_tiles) {
+      const int32_t* hu = hull_row + tid * 8;
+      a = (k0 < hu[1] && k0 + BN > hu[0]) || (k0 < hu[3] && k0 + BN > hu[2]);
+      u = (hu[4] <= k0 && k0 + BN <= hu[5]) || (hu[6] <= k0 && k0 + BN <= hu[7]);
+    }
+    if (w == 0) {
+      const unsigned long long am = __ballot(a), um = __ballot(u);
+      if (lane == 0) {
+        mask_lds[0] = am;
+        mask_lds[1] = um;
+      }
+    }
+  }
+  __syncthreads();
+  const unsigned long long act = mask_lds[0], unm = mask_lds[1];
+  const uint32_t act_lo = __builtin_amdgcn_readfirstlane((uint32_t)act);
+  const uint32_t act_hi = __builtin_amdgcn_readfirstlane((uint32_t)(act >> 32));
+  const unsigned long long act_mask = ((unsigned long long)act_hi << 32) | act_lo;
 
-      // per-row range, lse and delta of the tile's 64 queries
-      int4 my_rng = {0, 0, 0, 0};
-      float my_lse = INFINITY, my_delta = 0.0f;
-      if (tid < BM) {
-        const int ql = qt * BM + tid;
-        if (ql < seqlen_q) {
-          const int32_t* r = p.attn_range + q_begin + ql;
-          my_rng.x = r[0];
-          my_rng.y = max(min(r[p.total_q], seqlen_kv) - my_rng.x, 0);
-          if (p.n_ranges == 2) {
-            my_rng.z = r[2 * (int64_t)p.total_q];
-            my_rng.w = max(min(r[3 * (int64_t)p.total_q], seqlen_kv) - my_rng.z, 0);
-          }
-          my_lse = p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + ql] * kLog2e;
-          my_delta = p.delta[(int64_t)(q_begin + ql) * p.n_heads_q + head];
+  // the per-row range, lse and delta of a step's 64 queries: requested into registers
+  // (fetch_meta) while the previous step is being multiplied, parked in LDS (stash_meta)
+  // before the barrier that opens the step
+  int4 my_rng = {0, 0, 0, 0};
+  float my_lse = INFINITY, my_delta = 0.0f;
+  auto fetch_meta = [&](int head, int qt) {
+    my_rng = int4{0, 0, 0, 0};
+    my_lse = INFINITY;
+    my_delta = 0.0f;
+    if (tid < BM) {
+      const int ql = qt * BM + tid;
+      if (ql < seqlen_q) {
+        const int32_t* r = p.attn_range + q_begin + ql;
+        my_rng.x = r[0];
+        my_rng.y = max(min(r[p.total_q], seqlen_kv) - my_rng.x, 0);
+        if (p.n_ranges == 2) {
+          my_rng.z = r[2 * (int64_t)p.total_q];
+          my_rng.w = max(min(r[3 * (int64_t)p.total_q], seqlen_kv) - my_rng.z, 0);
         }
+        my_lse = p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + ql] * kLog2e;
+        my_delta = p.delta[(int64_t)(q_begin + ql) * p.n_heads_q + head];
       }
-      __syncthreads();  // previous tile fully consumed
-      // ---- Q and dO tiles: global -> LDS directly (rows past seqlen_q are masked below) ----
-      {
-        const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
-        Tile::load_async(lds_address(q_lds), q_base + off, goff, w);
-        Tile::load_async(lds_address(do_lds), do_base + off, goff, w);
-      }
-      if (tid < BM) {
-        *reinterpret_cast<int4*>(&rng_lds[tid * 4]) = my_rng;
-        lse_lds[tid] = my_lse;
-        delta_lds[tid] = my_delta;
-      }
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();
+    }
+  };
+  auto stash_meta = [&](int st) {
+    if (tid < BM) {
+      *reinterpret_cast<int4*>(&rng_lds[st][tid * 4]) = my_rng;
+      lse_lds[st][tid] = my_lse;
+      delta_lds[st][tid] = my_delta;
+    }
+  };
 
+  // steps: (q head of the group) x (active 64-query tile)
+  int hg = 0;
+  unsigned long long rem = act_mask;  // tiles of head hg still to do
+  int st = 0;
+  if (act_mask != 0 && group > 0) {
+    fetch_meta(kv_head * group, __builtin_ctzll(rem));
+    stash_meta(0);
+  }
+  while (act_mask != 0 && hg < group) {
+    const int head = kv_head * group + hg;
+    const int qt = __builtin_ctzll(rem);
+    const bool unmasked = (unm >> qt) & 1;
+    rem &= rem - 1;
+    int hg_next = hg;
+    if (rem == 0) {
+      rem = act_mask;
+      ++hg_next;
+    }
+    const bool more = hg_next < group;
+
+    __syncthreads();  // previous step fully consumed; this step's scalars are stashed
+    // ---- Q and dO tiles: global -> LDS directly (rows past seqlen_q are masked below) ----
+    {
+      const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
+      Tile::load_async(lds_address(q_lds), q_base + off, goff, w);
+      Tile::load_async(lds_address(do_lds), do_base + off, goff, w);
+    }
+    if (more) fetch_meta(kv_head * group + hg_next, __builtin_ctzll(rem));
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    {
       // ---- phase 1: S = Q K^T, dP = dO V^T on this wave's 32x32 sub-tile ---------------
       // the range mask enters S as the accumulator's initial value (0 / -inf)
       f32x16 s_acc, dp_acc;
@@ -301,7 +350,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       } else {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int4 rg = *reinterpret_cast<const int4*>(&rng_lds[(qi * 32 + acc_row(i, h)) * 4]);
+          const int4 rg = *reinterpret_cast<const int4*>(&rng_lds[st][(qi * 32 + acc_row(i, h)) * 4]);
           const bool ok = ((unsigned)(kv - rg.x) < (unsigned)rg.y) | ((unsigned)(kv - rg.z) < (unsigned)rg.w);
           s_acc[i] = ok ? 0.0f : -INFINITY;
         }
@@ -325,8 +374,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int qrow = qi * 32 + 8 * g + 4 * h;
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[qrow]);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[qrow]);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[st][qrow]);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][qrow]);
         float pv[4], dsv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -340,42 +389,49 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       }
       __syncthreads();  // P and dS of all four waves are in LDS
 
-      // ---- phase 2: this wave's dim slice ------------------------------------------------
-      // dV^T[dim, key] += dO^T[dim, q] P[q, key];  dK^T[dim, key] += Q^T[dim, q] dS[q, key]
+      // ---- phase 2 ---------------------------------------------------------------------------
+      // dV^T[dim, key] += dO^T[dim, q] P[q, key]   or   dK^T[dim, key] += Q^T[dim, q] dS[q, key]
       // (dO^T and Q^T come out of the row-major tiles by transpose loads)
+      {
+        const uint16_t* a_tile = is_dk ? q_lds : do_lds;
+        const uint16_t* b_rows = is_dk ? ds_lds : p_lds;
 #pragma unroll
-      for (int ks = 0; ks < BM / 16; ++ks) {
-        const u32x4 a_do = Tile::template read_col<false>(do_lds, col_rd, ks, 0);
-        const u32x4 a_q = Tile::template read_col<false>(q_lds, col_rd, ks, 0);
+        for (int ks = 0; ks < BM / 16; ++ks) {
+          u32x4 a[DB], bq[2];
 #pragma unroll
-        for (int u = 0; u < UPW; ++u) {
-          const int row = ((tile0 + u) * 32 + c) * T_STRIDE + ks * 16 + h * 8;
-          const u32x4 b_p = *reinterpret_cast<const u32x4*>(&p_lds[row]);
-          const u32x4 b_ds = *reinterpret_cast<const u32x4*>(&ds_lds[row]);
-          dv_acc[u] = mfma_32x32x16<DTYPE>(a_do, b_p, dv_acc[u]);
-          dk_acc[u] = mfma_32x32x16<DTYPE>(a_q, b_ds, dk_acc[u]);
+          for (int db = 0; db < DB; ++db) a[db] = Tile::template read_col<false>(a_tile, col_rd, ks, db);
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            bq[u] = *reinterpret_cast<const u32x4*>(&b_rows[(u * 32 + c) * T_STRIDE + ks * 16 + h * 8]);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) acc[db][u] = mfma_32x32x16<DTYPE>(a[db], bq[u], acc[db][u]);
         }
       }
     }
+    if (more) stash_meta(st ^ 1);
+    st ^= 1;
+    hg = hg_next;
   }
 
-  // ---- store dK, dV: lane = key, 4 consecutive dims per accumulator group ---------------
+  // ---- store dK or dV: lane = key, 4 consecutive dims per accumulator group ---------------
+  const float out_scale = is_dk ? p.scale : 1.0f;
+  uint16_t* dst = reinterpret_cast<uint16_t*>(is_dk ? p.dk : p.dv);
 #pragma unroll
-  for (int u = 0; u < UPW; ++u) {
+  for (int u = 0; u < 2; ++u) {
     const int64_t off = (int64_t)p.dkv_block_table[(int64_t)b * p.max_kv_blocks + blk] * p.dkv_slot_stride +
-                        (int64_t)(tok0 + (tile0 + u) * 32 + c) * p.dkv_token_stride + (int64_t)kv_head * D +
-                        slice * 32 + 4 * h;
-    uint16_t* dkp = reinterpret_cast<uint16_t*>(p.dk) + off;
-    uint16_t* dvp = reinterpret_cast<uint16_t*>(p.dv) + off;
+                        (int64_t)(tok0 + u * 32 + c) * p.dkv_token_stride + (int64_t)kv_head * D +
+                        dhalf * (D / 2) + 4 * h;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      u32x2 k4 = {pack2<DTYPE>(dk_acc[u][4 * g] * p.scale, dk_acc[u][4 * g + 1] * p.scale),
-                  pack2<DTYPE>(dk_acc[u][4 * g + 2] * p.scale, dk_acc[u][4 * g + 3] * p.scale)};
-      u32x2 v4 = {pack2<DTYPE>(dv_acc[u][4 * g], dv_acc[u][4 * g + 1]),
-                  pack2<DTYPE>(dv_acc[u][4 * g + 2], dv_acc[u][4 * g + 3])};
-      *reinterpret_cast<u32x2*>(dkp + 8 * g) = k4;
-      *reinterpret_cast<u32x2*>(dvp + 8 * g) = v4;
-    }
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& r = acc[db][u];
+        u32x2 v4 = {pack2<DTYPE>(r[4 * g] * out_scale, r[4 * g + 1] * out_scale),
+                    pack2<DTYPE>(r[4 * g + 2] * out_scale, r[4 * g + 3] * out_scale)};
+        *reinterpret_cast<u32x2*>(dst + off + db * 32 + 8 * g) = v4;
+      }
   }
 }
 
@@ -679,6 +735,8 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
   if (batch == 0) return DCP_OK;
   DCP_REQUIRE(block_size > 0 && block_size % kBwdBN == 0,
               "attn_bwd: block_size %d must be a positive multiple of %d", block_size, kBwdBN);
+  if (block_size > 64 * kBwdBM)
+    return fail(DCP_ERR_UNSUPPORTED, "attn_bwd: block_size %d unsupported (at most %d)", block_size, 64 * kBwdBM);
   DCP_REQUIRE(n_heads_q > 0 && n_heads_kv > 0 && n_heads_q % n_heads_kv == 0,
               "attn_bwd: n_heads_q %d must be a multiple of n_heads_kv %d", n_heads_q, n_heads_kv);
   DCP_REQUIRE(max_kv_blocks > 0 && n_out_slots > 0, "attn_bwd: empty block tables");
