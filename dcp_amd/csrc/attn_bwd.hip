@@ -178,7 +178,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // per k-step
   constexpr int DB = D / 64;  // 32-dim blocks per wave: 2 (D=128) or 1 (D=64)
 
-  __shared__ __attribute__((aligned(16))) uint16_t q_lds[Tile::SIZE];
+  // two stages of the Q tile (the next step's streams in during this step); LDS has no
+  // room for a second dO stage with two workgroups per CU, so dO is requested when its
+  // step opens and S = Q K^T is multiplied while it arrives
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds2[2][Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t do_lds[Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t p_lds[BN * T_STRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t ds_lds[BN * T_STRIDE];
@@ -313,8 +316,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   int hg = 0;
   unsigned long long rem = act_mask;  // tiles of head hg still to do
   int st = 0;
+  const uint32_t q_at = lds_address(&q_lds2[0][0]), do_at = lds_address(do_lds);
+  auto tile_off = [&](int head, int qt) -> int64_t { return (int64_t)qt * BM * q_row_stride + (int64_t)head * D; };
   if (act_mask != 0 && group > 0) {
-    fetch_meta(kv_head * group, __builtin_ctzll(rem));
+    const int qt0 = __builtin_ctzll(rem);
+    Tile::load_async(q_at, q_base + tile_off(kv_head * group, qt0), goff, w);
+    fetch_meta(kv_head * group, qt0);
     stash_meta(0);
   }
   while (act_mask != 0 && hg < group) {
@@ -329,16 +336,15 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
     const bool more = hg_next < group;
 
-    __syncthreads();  // previous step fully consumed; this step's scalars are stashed
-    // ---- Q and dO tiles: global -> LDS directly (rows past seqlen_q are masked below) ----
-    {
-      const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
-      Tile::load_async(lds_address(q_lds), q_base + off, goff, w);
-      Tile::load_async(lds_address(do_lds), do_base + off, goff, w);
-    }
-    if (more) fetch_meta(kv_head * group + hg_next, __builtin_ctzll(rem));
+    const uint16_t* q_lds = q_lds2[st];
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+    __syncthreads();  // previous step fully consumed; this step's Q tile and scalars are in LDS
+    // requests, oldest first: the next step's scalars, this step's dO tile, the next step's Q tile
+    const int qt_next = more ? __builtin_ctzll(rem) : 0;
+    if (more) fetch_meta(kv_head * group + hg_next, qt_next);
+    Tile::load_async(do_at, do_base + tile_off(head, qt), goff, w);
+    if (more)
+      Tile::load_async(q_at + (st ^ 1) * (Tile::SIZE * 2), q_base + tile_off(kv_head * group + hg_next, qt_next), goff, w);
     {
       // ---- phase 1: S = Q K^T, dP = dO V^T on this wave's 32x32 sub-tile ---------------
       // the range mask enters S as the accumulator's initial value (0 / -inf)
@@ -359,16 +365,23 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
 #pragma unroll
       for (int half = 0; half < KS / 4; ++half) {
-        u32x4 aq[4], ad[4];
+        u32x4 aq[4];
 #pragma unroll
         for (int k4 = 0; k4 < 4; ++k4) aq[k4] = Tile::read_row(q_lds, row_rd, 0, half * 4 + k4);
 #pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) s_acc = mfma_32x32x16<DTYPE>(aq[k4], kreg[half * 4 + k4], s_acc);
+      }
+      // the dO tile: everything requested before the next step's Q tile has to be in
+      if (more) __builtin_amdgcn_s_waitcnt(0x0F70 | Tile::LPW);  // vmcnt(LPW): only that Q tile may be pending
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+#pragma unroll
+      for (int half = 0; half < KS / 4; ++half) {
+        u32x4 ad[4];
+#pragma unroll
         for (int k4 = 0; k4 < 4; ++k4) ad[k4] = Tile::read_row(do_lds, row_rd, 0, half * 4 + k4);
 #pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) {
-          s_acc = mfma_32x32x16<DTYPE>(aq[k4], kreg[half * 4 + k4], s_acc);
-          dp_acc = mfma_32x32x16<DTYPE>(ad[k4], vreg[half * 4 + k4], dp_acc);
-        }
+        for (int k4 = 0; k4 < 4; ++k4) dp_acc = mfma_32x32x16<DTYPE>(ad[k4], vreg[half * 4 + k4], dp_acc);
       }
       // P, dS (lane = key 32ki + c; element i = query 32qi + acc_row(i,h)) -> LDS [key][query]
 #pragma unroll
