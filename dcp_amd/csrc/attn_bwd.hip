@@ -19,32 +19,28 @@
 // 64k-token causal schedule: device-scope float atomics from eight XCDs cost
 // more than the two recomputed products.
 //
-// dK/dV kernel, per (64 q) x (64 kv) tile.  Phase 1: wave (qi, ki) owns the
-// 32x32 sub-tile (queries 32qi.., keys 32ki..):
+// dK/dV kernel, per step of (64 q) x (64 kv).  Wave (qi, ki) owns the 32x32
+// sub-tile (queries 32qi.., keys 32ki..) from start to end:
 //
 //   S  = Q K^T          A = Q rows from LDS,   B = K held in registers
 //   dP = dO V^T         A = dO rows from LDS,  B = V held in registers
 //   P  = exp2(S*c - lse), dS = P * (dP - delta)   accumulator layout: lane =
 //                                                 key, 4 consecutive queries
 //                                                 per register group
-//   P, dS -> LDS as [key][query] with 8-byte stores
-//
-// Phase 2: each wave owns one of the two products for one half of the head dim
-// and all 64 keys, and contracts over the tile's 64 queries:
-//
 //   dV^T[dim, key] += dO^T P   A = dO^T: transpose-load from the row-major dO
-//                              tile, B = P rows from LDS
+//                              tile in accumulator row order, B = P straight
+//                              from the accumulators
 //   dK^T[dim, key] += Q^T dS   A = Q^T: transpose-load from the Q tile, B = dS
 //
-// so that every operand read from LDS feeds two MFMAs (a 2x2 block of
-// accumulators per k-step).
-//
-// Q and dO tiles go from global memory straight into LDS, row-major; nothing is
-// staged through registers or stored transposed.  The range mask enters S as
-// the accumulator's initial value (0 or -inf).  dK/dV of
-// a key never leave the workgroup's registers until the end, so the
-// per-(row, kv block) private dKV blocks of the plan need no atomics and are
-// written whole (zeros where no query of the row attends).
+// P and dS never leave the registers, so a step needs one workgroup barrier (the
+// one that publishes its tiles) and LDS holds nothing but the Q and dO tiles, two
+// stages of each: everything a step reads is requested one step ahead.  The two
+// waves that share a key half (qi = 0, 1) each hold a partial dK^T/dV^T over
+// their 32 queries; they are added once, after the loop, through LDS.  The range
+// mask enters S as the accumulator's initial value (0 or -inf).  dK/dV of a key
+// never leave the workgroup until the end, so the per-(row, kv block) private
+// dKV blocks of the plan need no atomics and are written whole (zeros where no
+// query of the row attends).
 #include <math.h>
 
 #include "attn_common.h"
@@ -165,41 +161,39 @@ __global__ __launch_bounds__(64) void bwd_tile_hull_kernel(const AttnBwdParams p
 }
 
 // ---------------------------------------------------------------------------
-// main kernel
+// dK/dV kernel
 // ---------------------------------------------------------------------------
 template <int DTYPE, int D>
 __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
   constexpr int BM = kBwdBM, BN = kBwdBN;
-  constexpr int KS = D / 16;        // k-steps over the head dim
-  constexpr int T_STRIDE = BM + 8;  // p_lds / ds_lds rows (elements): [key][query]
-  typedef KvTile<D> Tile;           // the Q and dO tiles: 64 queries x D
-  // second phase: a wave owns one of the two products (dV^T or dK^T) for one half of the
-  // head dim and all 64 keys: DB x 2 accumulator blocks that share DB + 2 operand reads
-  // per k-step
-  constexpr int DB = D / 64;  // 32-dim blocks per wave: 2 (D=128) or 1 (D=64)
+  constexpr int KS = D / 16;  // k-steps over the head dim
+  constexpr int DT = D / 32;  // 32-dim blocks of dK^T / dV^T
+  typedef KvTile<D> Tile;     // the Q and dO tiles: 64 queries x D
 
-  // two stages of the Q tile (the next step's streams in during this step); LDS has no
-  // room for a second dO stage with two workgroups per CU, so dO is requested when its
-  // step opens and S = Q K^T is multiplied while it arrives
-  __shared__ __attribute__((aligned(16))) uint16_t q_lds2[2][Tile::SIZE];
-  __shared__ __attribute__((aligned(16))) uint16_t do_lds[Tile::SIZE];
-  __shared__ __attribute__((aligned(16))) uint16_t p_lds[BN * T_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t ds_lds[BN * T_STRIDE];
-  // two stages of the per-query scalars: the next step's are fetched during this step
-  __shared__ __attribute__((aligned(16))) int rng_lds[2][BM * 4];
+  // two stages of everything a step reads: its Q and dO tiles and the per-query scalars.
+  // After the loop the tile area is reused (as floats) for the reduction over the two
+  // query halves.
+  __shared__ __attribute__((aligned(16))) uint16_t tiles[4][Tile::SIZE];  // [2 * stage + (0: Q, 1: dO)]
+  __shared__ __attribute__((aligned(16))) int rng_lds[2][4][BM];  // planes: start0, end0, start1, end1
   __shared__ __attribute__((aligned(16))) float lse_lds[2][BM];
   __shared__ __attribute__((aligned(16))) float delta_lds[2][BM];
   __shared__ unsigned long long mask_lds[2];
+  // With D = 128 the accumulators (128 registers), K and V (64) and the products in flight do
+  // not fit in 256 registers.  The compiler would spill to scratch memory, and a scratch
+  // reload waits for every outstanding global load, i.e. for the tiles requested a step
+  // ahead.  So the last VL k-steps of V are parked in LDS instead (per lane, read back with
+  // the other operands).
+  constexpr int VL = D == 128 ? 2 : 0;
+  __shared__ u32x4 v_park[VL > 0 ? kBwdThreads / 64 : 1][VL > 0 ? VL : 1][64];
+  static_assert(sizeof(tiles) >= 4 * 16 * DT * 64 * sizeof(float), "reduction buffer");
 
   const int tid = threadIdx.x;
-  const int w = tid >> 6;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int c = lane & 31;
   const int h = lane >> 5;
-  const int qi = w >> 1;  // query sub-tile of this wave in phase 1
-  const int ki = w & 1;   // key sub-tile of this wave in phase 1
-  const bool is_dk = (w & 1) != 0;  // phase 2: this wave accumulates dK^T (else dV^T) ...
-  const int dhalf = w >> 1;         // ... for dims [dhalf * D/2, (dhalf + 1) * D/2)
+  const int qi = w >> 1;  // this wave's 32 queries of a step
+  const int ki = w & 1;   // this wave's 32 keys of the tile
 
   // ---- which (row, kv head, key tile) ------------------------------------------
   // the key tiles of a row share its Q/dO tiles: keep them on one XCD
@@ -226,35 +220,36 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
                               (int64_t)tok0 * p.kv_token_stride + (int64_t)kv_head * D;
 
   // ---- K, V of this wave's 32 keys as B operands (lane = key, slots = dims) ------
-  u32x4 kreg[KS], vreg[KS];
+  u32x4 kreg[KS], vreg[KS - VL];
   {
     const int64_t off = kv_tile_off + (int64_t)(ki * 32 + c) * p.kv_token_stride + h * 8;
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k) + off;
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v) + off;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      kreg[ks] = *reinterpret_cast<const u32x4*>(kp + ks * 16);
-      vreg[ks] = *reinterpret_cast<const u32x4*>(vp + ks * 16);
-    }
+    for (int ks = 0; ks < KS; ++ks) kreg[ks] = *reinterpret_cast<const u32x4*>(kp + ks * 16);
+#pragma unroll
+    for (int ks = 0; ks < KS - VL; ++ks) vreg[ks] = *reinterpret_cast<const u32x4*>(vp + ks * 16);
+#pragma unroll
+    for (int j = 0; j < VL; ++j) v_park[w][j][lane] = *reinterpret_cast<const u32x4*>(vp + (KS - VL + j) * 16);
   }
 
-  // dK^T or dV^T of (dim block db of this wave's half) x (key tile u)
-  f32x16 acc[DB][2];
+  // this wave's share of dK^T and dV^T: (all dims) x (its 32 keys), summed over its query half
+  f32x16 dk_acc[DT], dv_acc[DT];
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[db][u][i] = 0.0f;
+    for (int i = 0; i < 16; ++i) {
+      dk_acc[dt][i] = 0.0f;
+      dv_acc[dt][i] = 0.0f;
+    }
 
   const int32_t* hull_row = p.hull + (int64_t)b * p.q_tiles_per_row * 8;
   // loop-invariant per-lane pieces of the addresses used in the loop
-  uint32_t goff[Tile::LPW];
-  Tile::lane_offsets(goff, q_row_stride, w, lane);
   const int row_rd = Tile::row_base(c, h) + qi * Tile::ROW32;
-  const int col_rd = Tile::col_base(lane, false) + dhalf * (D / 2);
+  const int col_rd = Tile::col_base(lane, true) + qi * Tile::ROW32;
   const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.block_size * q_row_stride;
   const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.block_size * q_row_stride;
+  const uint32_t tiles_at = lds_address(&tiles[0][0]);
 
   // ---- which 64-query tiles of the row see these keys (the same for every head) ----------
   // bit qt of `act`: some row of tile qt sees some key of the tile; of `unm`: every row sees
@@ -280,35 +275,33 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const uint32_t act_hi = __builtin_amdgcn_readfirstlane((uint32_t)(act >> 32));
   const unsigned long long act_mask = ((unsigned long long)act_hi << 32) | act_lo;
 
-  // the per-row range, lse and delta of a step's 64 queries: requested into registers
-  // (fetch_meta) while the previous step is being multiplied, parked in LDS (stash_meta)
-  // before the barrier that opens the step
-  int4 my_rng = {0, 0, 0, 0};
-  float my_lse = INFINITY, my_delta = 0.0f;
-  auto fetch_meta = [&](int head, int qt) {
-    my_rng = int4{0, 0, 0, 0};
-    my_lse = INFINITY;
-    my_delta = 0.0f;
-    if (tid < BM) {
-      const int ql = qt * BM + tid;
-      if (ql < seqlen_q) {
-        const int32_t* r = p.attn_range + q_begin + ql;
-        my_rng.x = r[0];
-        my_rng.y = max(min(r[p.total_q], seqlen_kv) - my_rng.x, 0);
-        if (p.n_ranges == 2) {
-          my_rng.z = r[2 * (int64_t)p.total_q];
-          my_rng.w = max(min(r[3 * (int64_t)p.total_q], seqlen_kv) - my_rng.z, 0);
-        }
-        my_lse = p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + ql] * kLog2e;
-        my_delta = p.delta[(int64_t)(q_begin + ql) * p.n_heads_q + head];
+  // Everything step (head, qt) reads is requested a step ahead, straight into LDS stage st
+  // and with nothing held in registers meanwhile: the Q and dO tiles, and one value per
+  // query of the range planes (waves 0 and 1), lse (wave 2) and delta (wave 3).  Queries
+  // past seqlen_q read the last valid query's values; they are masked where they are used.
+  const uint32_t rng_at = lds_address(&rng_lds[0][0][0]), lse_at = lds_address(&lse_lds[0][0]),
+                 delta_at = lds_address(&delta_lds[0][0]);
+  auto request = [&](int head, int qt, int st) {
+    // the per-lane offsets are recomputed per step on purpose: the registers that would
+    // hold them across the step are needed for the accumulators
+    int lane_now = lane;
+    asm volatile("" : "+v"(lane_now));
+    uint32_t goff[Tile::LPW];
+    Tile::lane_offsets(goff, q_row_stride, w, lane_now);
+    const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
+    Tile::load_async(tiles_at + (2 * st) * (Tile::SIZE * 2), q_base + off, goff, w);
+    Tile::load_async(tiles_at + (2 * st + 1) * (Tile::SIZE * 2), do_base + off, goff, w);
+    const int ql = min(qt * BM + lane, seqlen_q - 1);
+    if (w < 2) {
+      if (w == 0 || p.n_ranges == 2) {
+        const int32_t* r = p.attn_range + (int64_t)(2 * w) * p.total_q + q_begin + ql;
+        load_async_dword(rng_at + ((st * 4 + 2 * w) * BM) * 4, r);
+        load_async_dword(rng_at + ((st * 4 + 2 * w + 1) * BM) * 4, r + p.total_q);
       }
-    }
-  };
-  auto stash_meta = [&](int st) {
-    if (tid < BM) {
-      *reinterpret_cast<int4*>(&rng_lds[st][tid * 4]) = my_rng;
-      lse_lds[st][tid] = my_lse;
-      delta_lds[st][tid] = my_delta;
+    } else if (w == 2) {
+      load_async_dword(lse_at + st * BM * 4, p.lse + ((int64_t)head * p.n_out_slots + o_slot) * p.block_size + ql);
+    } else {
+      load_async_dword(delta_at + st * BM * 4, p.delta + (int64_t)(q_begin + ql) * p.n_heads_q + head);
     }
   };
 
@@ -316,16 +309,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   int hg = 0;
   unsigned long long rem = act_mask;  // tiles of head hg still to do
   int st = 0;
-  const uint32_t q_at = lds_address(&q_lds2[0][0]), do_at = lds_address(do_lds);
-  auto tile_off = [&](int head, int qt) -> int64_t { return (int64_t)qt * BM * q_row_stride + (int64_t)head * D; };
-  if (act_mask != 0 && group > 0) {
-    const int qt0 = __builtin_ctzll(rem);
-    Tile::load_async(q_at, q_base + tile_off(kv_head * group, qt0), goff, w);
-    fetch_meta(kv_head * group, qt0);
-    stash_meta(0);
-  }
+  if (act_mask != 0 && group > 0) request(kv_head * group, __builtin_ctzll(rem), 0);
   while (act_mask != 0 && hg < group) {
-    const int head = kv_head * group + hg;
     const int qt = __builtin_ctzll(rem);
     const bool unmasked = (unm >> qt) & 1;
     rem &= rem - 1;
@@ -336,116 +321,126 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
     const bool more = hg_next < group;
 
-    const uint16_t* q_lds = q_lds2[st];
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // previous step fully consumed; this step's Q tile and scalars are in LDS
-    // requests, oldest first: the next step's scalars, this step's dO tile, the next step's Q tile
-    const int qt_next = more ? __builtin_ctzll(rem) : 0;
-    if (more) fetch_meta(kv_head * group + hg_next, qt_next);
-    Tile::load_async(do_at, do_base + tile_off(head, qt), goff, w);
-    if (more)
-      Tile::load_async(q_at + (st ^ 1) * (Tile::SIZE * 2), q_base + tile_off(kv_head * group + hg_next, qt_next), goff, w);
-    {
-      // ---- phase 1: S = Q K^T, dP = dO V^T on this wave's 32x32 sub-tile ---------------
-      // the range mask enters S as the accumulator's initial value (0 / -inf)
-      f32x16 s_acc, dp_acc;
-      const int kv = k0 + ki * 32 + c;
-      if (unmasked) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int4 rg = *reinterpret_cast<const int4*>(&rng_lds[st][(qi * 32 + acc_row(i, h)) * 4]);
-          const bool ok = ((unsigned)(kv - rg.x) < (unsigned)rg.y) | ((unsigned)(kv - rg.z) < (unsigned)rg.w);
-          s_acc[i] = ok ? 0.0f : -INFINITY;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
-#pragma unroll
-      for (int half = 0; half < KS / 4; ++half) {
-        u32x4 aq[4];
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) aq[k4] = Tile::read_row(q_lds, row_rd, 0, half * 4 + k4);
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) s_acc = mfma_32x32x16<DTYPE>(aq[k4], kreg[half * 4 + k4], s_acc);
-      }
-      // the dO tile: everything requested before the next step's Q tile has to be in
-      if (more) __builtin_amdgcn_s_waitcnt(0x0F70 | Tile::LPW);  // vmcnt(LPW): only that Q tile may be pending
-      else __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
-#pragma unroll
-      for (int half = 0; half < KS / 4; ++half) {
-        u32x4 ad[4];
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) ad[k4] = Tile::read_row(do_lds, row_rd, 0, half * 4 + k4);
-#pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) dp_acc = mfma_32x32x16<DTYPE>(ad[k4], vreg[half * 4 + k4], dp_acc);
-      }
-      // P, dS (lane = key 32ki + c; element i = query 32qi + acc_row(i,h)) -> LDS [key][query]
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int qrow = qi * 32 + 8 * g + 4 * h;
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[st][qrow]);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][qrow]);
-        float pv[4], dsv[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));  // masked: exp2(-inf) = 0
-          dsv[r] = pv[r] * (dp_acc[4 * g + r] - d4[r]);
-        }
-        u32x2 p4 = {pack2<DTYPE>(pv[0], pv[1]), pack2<DTYPE>(pv[2], pv[3])};
-        u32x2 s4 = {pack2<DTYPE>(dsv[0], dsv[1]), pack2<DTYPE>(dsv[2], dsv[3])};
-        *reinterpret_cast<u32x2*>(&p_lds[(ki * 32 + c) * T_STRIDE + qrow]) = p4;
-        *reinterpret_cast<u32x2*>(&ds_lds[(ki * 32 + c) * T_STRIDE + qrow]) = s4;
-      }
-      __syncthreads();  // P and dS of all four waves are in LDS
+    __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed
+    if (more) request(kv_head * group + hg_next, __builtin_ctzll(rem), st ^ 1);
+    const uint16_t* q_lds = tiles[2 * st];
+    const uint16_t* do_lds = tiles[2 * st + 1];
 
-      // ---- phase 2 ---------------------------------------------------------------------------
-      // dV^T[dim, key] += dO^T[dim, q] P[q, key]   or   dK^T[dim, key] += Q^T[dim, q] dS[q, key]
-      // (dO^T and Q^T come out of the row-major tiles by transpose loads)
-      {
-        const uint16_t* a_tile = is_dk ? q_lds : do_lds;
-        const uint16_t* b_rows = is_dk ? ds_lds : p_lds;
+    // ---- S = Q K^T, dP = dO V^T on this wave's 32 queries x 32 keys --------------------
+    // (A = rows of the Q / dO tile, B = K / V in registers; lane = key, element i = query
+    // 32qi + acc_row(i, h)).  The range mask enters S as the accumulator's initial value.
+    f32x16 s_acc, dp_acc;
+    const int kv = k0 + ki * 32 + c;
+    if (unmasked) {
 #pragma unroll
-        for (int ks = 0; ks < BM / 16; ++ks) {
-          u32x4 a[DB], bq[2];
+      for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
+    } else {
 #pragma unroll
-          for (int db = 0; db < DB; ++db) a[db] = Tile::template read_col<false>(a_tile, col_rd, ks, db);
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-            bq[u] = *reinterpret_cast<const u32x4*>(&b_rows[(u * 32 + c) * T_STRIDE + ks * 16 + h * 8]);
-#pragma unroll
-          for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int u = 0; u < 2; ++u) acc[db][u] = mfma_32x32x16<DTYPE>(a[db], bq[u], acc[db][u]);
+      for (int i = 0; i < 16; ++i) {
+        const int r = qi * 32 + acc_row(i, h);
+        const int s0 = rng_lds[st][0][r], len0 = min(rng_lds[st][1][r], seqlen_kv) - s0;
+        bool ok = (unsigned)(kv - s0) < (unsigned)max(len0, 0);
+        if (p.n_ranges == 2) {
+          const int s1 = rng_lds[st][2][r], len1 = min(rng_lds[st][3][r], seqlen_kv) - s1;
+          ok |= (unsigned)(kv - s1) < (unsigned)max(len1, 0);
         }
+        ok &= qt * BM + r < seqlen_q;
+        s_acc[i] = ok ? 0.0f : -INFINITY;
       }
     }
-    if (more) stash_meta(st ^ 1);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
+    {
+      // operands are read one k-step ahead of their MFMAs, two k-steps' worth at most live
+      u32x4 aq[2], ad[2];
+      aq[0] = Tile::read_row(q_lds, row_rd, 0, 0);
+      ad[0] = Tile::read_row(do_lds, row_rd, 0, 0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) {
+          aq[(ks + 1) & 1] = Tile::read_row(q_lds, row_rd, 0, ks + 1);
+          ad[(ks + 1) & 1] = Tile::read_row(do_lds, row_rd, 0, ks + 1);
+        }
+        s_acc = mfma_32x32x16<DTYPE>(aq[ks & 1], kreg[ks], s_acc);
+        if (ks < KS - VL) dp_acc = mfma_32x32x16<DTYPE>(ad[ks & 1], vreg[ks], dp_acc);
+        else dp_acc = mfma_32x32x16<DTYPE>(ad[ks & 1], v_park[w][VL > 0 ? ks - (KS - VL) : 0][lane], dp_acc);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from piling up in registers
+      }
+    }
+    // ---- P = exp2(S c - lse), dS = P (dP - delta), packed in accumulator order: as B operands
+    // they feed the next products without leaving the registers -------------------------------
+    u32x4 pb[2], dsb[2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int qrow = qi * 32 + 8 * g + 4 * h;
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[st][qrow]);
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][qrow]);
+      float pv[4], dsv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -kLog2e * l4[r]));  // masked: exp2(-inf) = 0
+        dsv[r] = pv[r] * (dp_acc[4 * g + r] - d4[r]);
+      }
+      pb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(pv[0], pv[1]);
+      pb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(pv[2], pv[3]);
+      dsb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(dsv[0], dsv[1]);
+      dsb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(dsv[2], dsv[3]);
+    }
+    // ---- dV^T[dim, key] += dO^T[dim, q] P[q, key];  dK^T[dim, key] += Q^T[dim, q] dS[q, key]
+    // over this wave's 32 queries (dO^T and Q^T come out of the row-major tiles by
+    // transpose loads, in the accumulators' row order) -----------------------------------------
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+      for (int d2 = 0; d2 < DT; d2 += 2) {
+        u32x4 a_do[2], a_q[2];
+#pragma unroll
+        for (int j = 0; j < 2 && d2 + j < DT; ++j) a_do[j] = Tile::template read_col<true>(do_lds, col_rd, s2, d2 + j);
+#pragma unroll
+        for (int j = 0; j < 2 && d2 + j < DT; ++j) a_q[j] = Tile::template read_col<true>(q_lds, col_rd, s2, d2 + j);
+#pragma unroll
+        for (int j = 0; j < 2 && d2 + j < DT; ++j) {
+          dv_acc[d2 + j] = mfma_32x32x16<DTYPE>(a_do[j], pb[s2], dv_acc[d2 + j]);
+          dk_acc[d2 + j] = mfma_32x32x16<DTYPE>(a_q[j], dsb[s2], dk_acc[d2 + j]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     st ^= 1;
     hg = hg_next;
   }
 
-  // ---- store dK or dV: lane = key, 4 consecutive dims per accumulator group ---------------
-  const float out_scale = is_dk ? p.scale : 1.0f;
-  uint16_t* dst = reinterpret_cast<uint16_t*>(is_dk ? p.dk : p.dv);
+  // ---- sum the two query halves: the qi = 0 waves finish dV, the qi = 1 waves dK; each
+  // wave hands the other product to its partner (same keys) through LDS ----------------------
+  __syncthreads();  // nobody reads the tiles any more
+  float* red = reinterpret_cast<float*>(&tiles[0][0]) + w * (16 * DT * 64);
+  {
+    const f32x16* give = qi == 0 ? dk_acc : dv_acc;
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int64_t off = (int64_t)p.dkv_block_table[(int64_t)b * p.max_kv_blocks + blk] * p.dkv_slot_stride +
-                        (int64_t)(tok0 + u * 32 + c) * p.dkv_token_stride + (int64_t)kv_head * D +
-                        dhalf * (D / 2) + 4 * h;
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x16& r = acc[db][u];
-        u32x2 v4 = {pack2<DTYPE>(r[4 * g] * out_scale, r[4 * g + 1] * out_scale),
-                    pack2<DTYPE>(r[4 * g + 2] * out_scale, r[4 * g + 3] * out_scale)};
-        *reinterpret_cast<u32x2*>(dst + off + db * 32 + 8 * g) = v4;
-      }
+      for (int i = 0; i < 16; ++i) red[(dt * 16 + i) * 64 + lane] = qi == 0 ? dk_acc[dt][i] : dv_acc[dt][i];
+    (void)give;
   }
+  __syncthreads();
+  const float* take = reinterpret_cast<const float*>(&tiles[0][0]) + (w ^ 2) * (16 * DT * 64);
+  const float out_scale = qi == 0 ? 1.0f : p.scale;
+  uint16_t* dst = reinterpret_cast<uint16_t*>(qi == 0 ? p.dv : p.dk);
+  const int64_t off = (int64_t)p.dkv_block_table[(int64_t)b * p.max_kv_blocks + blk] * p.dkv_slot_stride +
+                      (int64_t)(tok0 + ki * 32 + c) * p.dkv_token_stride + (int64_t)kv_head * D + 4 * h;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float r[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        r[j] = ((qi == 0 ? dv_acc[dt][i] : dk_acc[dt][i]) + take[(dt * 16 + i) * 64 + lane]) * out_scale;
+      }
+      u32x2 v4 = {pack2<DTYPE>(r[0], r[1]), pack2<DTYPE>(r[2], r[3])};
+      *reinterpret_cast<u32x2*>(dst + off + dt * 32 + 8 * g) = v4;
+    }
 }
 
 // ---------------------------------------------------------------------------

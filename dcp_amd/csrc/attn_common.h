@@ -105,6 +105,15 @@ __device__ __forceinline__ uint32_t lds_address(T* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)p;
 }
 
+// One 4-byte element per lane from global memory straight into LDS: lane l's value lands
+// at lds_at + 4*l (lds_at wave-uniform).  Ordered by the caller like the tile loads below.
+__device__ __forceinline__ void load_async_dword(uint32_t lds_at, const void* g) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_at)), "v"(g)
+               : "memory");
+}
+
 template <int D, int NW = 4>
 struct KvTile {
   static constexpr int ROWS = 64;
