@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # cannot be read from inside the benchmark, so the figure is per workload and is only
 # reported for the workload it was measured on.
 MEASURED_TRAFFIC_BYTES = {
-    "llama3_8b_causal_64k": int(((1409263.8 + 1856554.1) * 2.0 + (1302542.9 + 581640.1) * 1.0) * 1024),
+    "llama3_8b_causal_64k": int(((1360743.7 + 1958567.1) * 2.0 + (1302549.4 + 581657.4) * 1.0) * 1024),
 }
 
 
