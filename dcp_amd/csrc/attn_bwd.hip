@@ -281,16 +281,17 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // past seqlen_q read the last valid query's values; they are masked where they are used.
   const uint32_t rng_at = lds_address(&rng_lds[0][0][0]), lse_at = lds_address(&lse_lds[0][0]),
                  delta_at = lds_address(&delta_lds[0][0]);
-  auto request = [&](int head, int qt, int st) {
-    // the per-lane offsets are recomputed per step on purpose: the registers that would
-    // hold them across the step are needed for the accumulators
-    int lane_now = lane;
-    asm volatile("" : "+v"(lane_now));
-    uint32_t goff[Tile::LPW];
-    Tile::lane_offsets(goff, q_row_stride, w, lane_now);
+  const uint32_t goff0 = Tile::lane_offset0(q_row_stride, w, lane);
+  // tile load idx of a step: the wave's group loads of the Q tile, then of the dO tile
+  constexpr int NL = 2 * Tile::LPW;
+  static_assert(NL <= KS, "half of the tile loads go between the k-steps of the first phase");
+  auto request_tile = [&](int idx, int head, int qt, int st) {
     const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
-    Tile::load_async(tiles_at + (2 * st) * (Tile::SIZE * 2), q_base + off, goff, w);
-    Tile::load_async(tiles_at + (2 * st + 1) * (Tile::SIZE * 2), do_base + off, goff, w);
+    const bool is_do = idx >= Tile::LPW;
+    Tile::load_group(tiles_at + (2 * st + (is_do ? 1 : 0)) * (Tile::SIZE * 2), (is_do ? do_base : q_base) + off, goff0,
+                     q_row_stride, w, is_do ? idx - Tile::LPW : idx);
+  };
+  auto request_scalars = [&](int head, int qt, int st) {
     const int ql = min(qt * BM + lane, seqlen_q - 1);
     if (w < 2) {
       if (w == 0 || p.n_ranges == 2) {
@@ -309,7 +310,16 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   int hg = 0;
   unsigned long long rem = act_mask;  // tiles of head hg still to do
   int st = 0;
-  if (act_mask != 0 && group > 0) request(kv_head * group, __builtin_ctzll(rem), 0);
+  if (act_mask != 0 && group > 0) {
+    request_scalars(kv_head * group, __builtin_ctzll(rem), 0);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) request_tile(i, kv_head * group, __builtin_ctzll(rem), 0);
+#ifdef DCP_EXP_NOLOADS
+    request_scalars(kv_head * group, __builtin_ctzll(rem), 1);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) request_tile(i, kv_head * group, __builtin_ctzll(rem), 1);
+#endif
+  }
   while (act_mask != 0 && hg < group) {
     const int qt = __builtin_ctzll(rem);
     const bool unmasked = (unm >> qt) & 1;
@@ -319,11 +329,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       rem = act_mask;
       ++hg_next;
     }
+#ifdef DCP_EXP_NOLOADS
+    const bool more = false;
+#else
     const bool more = hg_next < group;
+#endif
 
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed
-    if (more) request(kv_head * group + hg_next, __builtin_ctzll(rem), st ^ 1);
+    // the next step's tiles are requested one load per k-step below: a burst here would
+    // hold the wave at its last load until the memory pipeline has taken them all
+    const int head_next = kv_head * group + hg_next, qt_next = __builtin_ctzll(rem);
+    if (more) request_scalars(head_next, qt_next, st ^ 1);
     const uint16_t* q_lds = tiles[2 * st];
     const uint16_t* do_lds = tiles[2 * st + 1];
 
@@ -365,6 +382,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         s_acc = mfma_32x32x16<DTYPE>(aq[ks & 1], kreg[ks], s_acc);
         if (ks < KS - VL) dp_acc = mfma_32x32x16<DTYPE>(ad[ks & 1], vreg[ks], dp_acc);
         else dp_acc = mfma_32x32x16<DTYPE>(ad[ks & 1], v_park[w][VL > 0 ? ks - (KS - VL) : 0][lane], dp_acc);
+        if (ks % 2 == 0 && ks / 2 < NL / 2 && more) request_tile(ks / 2, head_next, qt_next, st ^ 1);
         __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from piling up in registers
       }
     }
@@ -403,6 +421,13 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         for (int j = 0; j < 2 && d2 + j < DT; ++j) {
           dv_acc[d2 + j] = mfma_32x32x16<DTYPE>(a_do[j], pb[s2], dv_acc[d2 + j]);
           dk_acc[d2 + j] = mfma_32x32x16<DTYPE>(a_q[j], dsb[s2], dk_acc[d2 + j]);
+        }
+        {
+          constexpr int GROUPS = 2 * ((DT + 1) / 2), PER = (NL / 2 + GROUPS - 1) / GROUPS;
+          const int grp = s2 * ((DT + 1) / 2) + d2 / 2;
+#pragma unroll
+          for (int i = grp * PER; i < (grp + 1) * PER && i < NL / 2; ++i)
+            if (more) request_tile(NL / 2 + i, head_next, qt_next, st ^ 1);
         }
         __builtin_amdgcn_sched_barrier(0);
       }

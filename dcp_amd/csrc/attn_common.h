@@ -168,6 +168,29 @@ struct KvTile {
                    : "memory");
     }
   }
+  // The same loads one at a time, so that a kernel can spread them between its matrix
+  // instructions instead of issuing a burst (a burst fills the memory pipeline's queue
+  // and the wave sits at the last load until the queue drains).  The rows of group
+  // load i lie 4*i rows below those of group load 0, so one per-lane byte offset
+  // (lane_offset0) serves all of them and the rest of the address is wave-uniform:
+  // scalar base + vector offset addressing, no per-load address arithmetic.
+  __device__ static __forceinline__ uint32_t lane_offset0(int64_t row_stride, int wave, int lane) {
+    constexpr int CH = D / 8;
+    static_assert((LPW & (LPW - 1)) == 0 && LPW <= 4, "group loads of a wave must not carry into grp >> 2");
+    return (uint32_t)((row_of(wave * LPW, lane / CH) * row_stride + (lane % CH) * 8) * 2);
+  }
+  // `g` (wave-uniform) points at (row 0, the head's first element) of the tile.
+  __device__ static __forceinline__ void load_group(uint32_t tile_at, const uint16_t* g, uint32_t off0,
+                                                    int64_t row_stride, int wave, int i) {
+    const uint32_t lds_at = __builtin_amdgcn_readfirstlane(tile_at + (wave * LPW + i) * GROUP_STRIDE * 2);
+    const uint64_t a = reinterpret_cast<uint64_t>(g) + (uint64_t)(i * 8) * (uint64_t)row_stride;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    const uint64_t base = ((uint64_t)hi << 32) | lo;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_at), "v"(off0), "s"(base)
+                 : "memory");
+  }
   // Row operand of lane (c, h): elements 16*ks + 8h.. of row 32*nt + c at
   //   tile + row_base(c, h) + nt*ROW32 + ks*16
   __device__ static __forceinline__ int row_base(int c, int h) { return at(c, 8 * h); }
