@@ -314,11 +314,6 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     request_scalars(kv_head * group, __builtin_ctzll(rem), 0);
 #pragma unroll
     for (int i = 0; i < NL; ++i) request_tile(i, kv_head * group, __builtin_ctzll(rem), 0);
-#ifdef DCP_EXP_NOLOADS
-    request_scalars(kv_head * group, __builtin_ctzll(rem), 1);
-#pragma unroll
-    for (int i = 0; i < NL; ++i) request_tile(i, kv_head * group, __builtin_ctzll(rem), 1);
-#endif
   }
   while (act_mask != 0 && hg < group) {
     const int qt = __builtin_ctzll(rem);
@@ -329,11 +324,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       rem = act_mask;
       ++hg_next;
     }
-#ifdef DCP_EXP_NOLOADS
-    const bool more = false;
-#else
     const bool more = hg_next < group;
-#endif
 
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed

@@ -298,8 +298,18 @@ struct TileCursor {
   int blk;      // block within the row
   int64_t off;  // element offset of the tile's first key row
 
+  // The two sources are read through volatile pointers so that the compiler keeps them as an
+  // LDS read and a global read under a (wave-uniform) branch: merged into one generic-address
+  // load, the read would be followed by a wait for every outstanding global load, i.e. for the
+  // tiles just requested.  The result is the same in every lane; readfirstlane moves it (and
+  // all the offset arithmetic that follows) to the scalar unit.
   __device__ __forceinline__ static int slot(const int* slot_lds, const int32_t* kv_table, int blk) {
-    return blk < kSlotTableCap ? slot_lds[blk] : kv_table[blk];
+    typedef __attribute__((address_space(3))) const volatile int lds_int;
+    typedef __attribute__((address_space(1))) const volatile int32_t global_int;
+    int v;
+    if (blk < kSlotTableCap) v = *(reinterpret_cast<lds_int*>(lds_address(slot_lds)) + blk);
+    else v = *((global_int*)kv_table + blk);
+    return __builtin_amdgcn_readfirstlane(v);
   }
   __device__ __forceinline__ void seek(const TileRuns& runs, int i, int tiles_per_block, const int* slot_lds,
                                        const int32_t* kv_table, int64_t slot_stride, int64_t tile_stride) {

@@ -66,13 +66,23 @@ struct AttnFwdParams {
   float scale_log2;  // softmax_scale * log2(e)
 };
 
-constexpr int kFwdBM = 128;
 constexpr int kFwdBN = 64;
 constexpr int kFwdThreads = 256;
+// The running maximum of a row is only raised (and O^T rescaled) when the tile's maximum
+// exceeds it by more than this many powers of two; until then the weights of the tile are
+// taken relative to the old maximum and are at most 2^kLazyMax.  With fp32 sums and
+// accumulators that costs no accuracy, and it takes the rescale (64 multiplies per query
+// block) out of almost every tile after a row's first few.
+constexpr float kLazyMax = 8.0f;
 
-template <int DTYPE, int D>
-__global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdParams p) {
+// QB = 32-row query blocks per wave: the workgroup owns 128*QB query rows.  With QB = 2 every
+// K / V^T operand read from LDS feeds two matrix instructions and every tile brought into LDS
+// serves twice the arithmetic; the wave then needs the whole register file (one workgroup
+// per CU, accumulators in the AGPR half).
+template <int DTYPE, int D, int QB>
+__global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
   constexpr int BN = kFwdBN;
+  constexpr int BM = 128 * QB;
   constexpr int KS = D / 16;  // k-steps of S^T = K Q^T
   constexpr int DT = D / 32;  // 32-row tiles of O^T
   typedef KvTile<D> KTile;  // read as rows (A operand of S^T)
@@ -87,7 +97,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   __shared__ int slot_lds[kSlotTableCap];
 
   const int tid = threadIdx.x;
-  const int w = tid >> 6;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int c = lane & 31;
   const int h = lane >> 5;
@@ -104,49 +114,61 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   const int q_begin = p.cu_seqlens_q[b];
   const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
   const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
-  if (qt * kFwdBM >= seqlen_q) return;
+  if (qt * BM >= seqlen_q) return;
   const int kv_head = head / (p.n_heads_q / p.n_heads_kv);
   const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
 
-  const int q_local = qt * kFwdBM + w * 32 + c;
-  const bool q_valid = q_local < seqlen_q;
+  int q_local[QB];
+  bool q_valid[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    q_local[qb] = qt * BM + (w * QB + qb) * 32 + c;
+    q_valid[qb] = q_local[qb] < seqlen_q;
+  }
 
-  // ---- Q fragment (B operand of S^T) ---------------------------------------
-  u32x4 qreg[KS];
-  {
+  // ---- Q fragments (B operands of S^T) -------------------------------------
+  u32x4 qreg[QB][KS];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
     const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) +
-                         ((int64_t)p.q_block_table[b] * p.block_size + q_local) * q_row_stride +
+                         ((int64_t)p.q_block_table[b] * p.block_size + q_local[qb]) * q_row_stride +
                          (int64_t)head * D + h * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 z = {0, 0, 0, 0};
-      qreg[ks] = q_valid ? *reinterpret_cast<const u32x4*>(qp + ks * 16) : z;
+      qreg[qb][ks] = q_valid[qb] ? *reinterpret_cast<const u32x4*>(qp + ks * 16) : z;
     }
   }
 
-  // ---- this lane's query row: ranges ---------------------------------------
-  RangePair rng = {0, 0, 0, 0};
-  if (q_valid) {
-    const int32_t* r = p.attn_range + q_begin + q_local;
-    const int s0 = r[0], e0 = min(r[p.total_q], seqlen_kv);
-    rng.s0 = s0;
-    rng.len0 = max(e0 - s0, 0);
-    if (p.n_ranges == 2) {
-      const int s1 = r[2 * (int64_t)p.total_q], e1 = min(r[3 * (int64_t)p.total_q], seqlen_kv);
-      rng.s1 = s1;
-      rng.len1 = max(e1 - s1, 0);
-    }
-  }
-  // hull (what any row of the wave can see) and core (what every row sees)
+  // ---- this lane's query rows: ranges --------------------------------------
+  RangePair rng[QB];
   const int big = 0x7fffffff;
-  const int w_lo0 = wave_min(rng.len0 > 0 ? rng.s0 : big);
-  const int w_hi0 = wave_max(rng.len0 > 0 ? rng.s0 + rng.len0 : 0);
-  const int w_lo1 = wave_min(rng.len1 > 0 ? rng.s1 : big);
-  const int w_hi1 = wave_max(rng.len1 > 0 ? rng.s1 + rng.len1 : 0);
-  const int core_lo0 = wave_max(rng.len0 > 0 ? rng.s0 : big);
-  const int core_hi0 = wave_min(rng.len0 > 0 ? rng.s0 + rng.len0 : 0);
-  const int core_lo1 = wave_max(rng.len1 > 0 ? rng.s1 : big);
-  const int core_hi1 = wave_min(rng.len1 > 0 ? rng.s1 + rng.len1 : 0);
+  int w_lo0 = big, w_hi0 = 0, w_lo1 = big, w_hi1 = 0;            // hull: what any row of the wave can see
+  int core_lo0 = 0, core_hi0 = big, core_lo1 = 0, core_hi1 = big;  // core: what every row sees
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    RangePair r4 = {0, 0, 0, 0};
+    if (q_valid[qb]) {
+      const int32_t* r = p.attn_range + q_begin + q_local[qb];
+      const int s0 = r[0], e0 = min(r[p.total_q], seqlen_kv);
+      r4.s0 = s0;
+      r4.len0 = max(e0 - s0, 0);
+      if (p.n_ranges == 2) {
+        const int s1 = r[2 * (int64_t)p.total_q], e1 = min(r[3 * (int64_t)p.total_q], seqlen_kv);
+        r4.s1 = s1;
+        r4.len1 = max(e1 - s1, 0);
+      }
+    }
+    rng[qb] = r4;
+    w_lo0 = min(w_lo0, wave_min(r4.len0 > 0 ? r4.s0 : big));
+    w_hi0 = max(w_hi0, wave_max(r4.len0 > 0 ? r4.s0 + r4.len0 : 0));
+    w_lo1 = min(w_lo1, wave_min(r4.len1 > 0 ? r4.s1 : big));
+    w_hi1 = max(w_hi1, wave_max(r4.len1 > 0 ? r4.s1 + r4.len1 : 0));
+    core_lo0 = max(core_lo0, wave_max(r4.len0 > 0 ? r4.s0 : big));
+    core_hi0 = min(core_hi0, wave_min(r4.len0 > 0 ? r4.s0 + r4.len0 : 0));
+    core_lo1 = max(core_lo1, wave_max(r4.len1 > 0 ? r4.s1 : big));
+    core_hi1 = min(core_hi1, wave_min(r4.len1 > 0 ? r4.s1 + r4.len1 : 0));
+  }
   const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
   load_slot_table(slot_lds, kv_table, p.max_kv_blocks, tid, kFwdThreads);
   if (lane == 0) {
@@ -168,21 +190,25 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   const int n_tiles = runs.count();
 
   // ---- running state ---------------------------------------------------------
-  f32x16 o_acc[DT];
+  f32x16 o_acc[QB][DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) o_acc[dt][i] = 0.0f;
-  float m_run = -INFINITY;  // running max, log2 domain
-  float l_run = 0.0f;       // this half-wave's partial row sum
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o_acc[qb][dt][i] = 0.0f;
+  float m_run[QB], l_run[QB];  // reference maximum (log2 domain); this half-wave's partial row sum
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.0f;
+  }
 
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
 
   // loop-invariant per-lane pieces of every address used in the key loop
-  uint32_t k_goff[KTile::LPW], v_goff[VTile::LPW];
-  KTile::lane_offsets(k_goff, p.kv_token_stride, w, lane);
-  VTile::lane_offsets(v_goff, p.kv_token_stride, w, lane);
+  const uint32_t kv_goff0 = KTile::lane_offset0(p.kv_token_stride, w, lane);
   const int k_rd = KTile::row_base(c, h);
   const int v_rd = VTile::col_base(lane, true);
 
@@ -207,26 +233,51 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
     const int k0 = tile * BN;
     return (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
   };
+  // the same test in tile numbers, for the loop's fast path: tiles [full0, full0 + n_full0) and
+  // [full1, full1 + n_full1) lie inside every row's range
+  const int full0 = (core_lo0 > big - BN ? big / BN : (core_lo0 + BN - 1) / BN), n_full0 = max(core_hi0 / BN - full0, 0);
+  const int full1 = (core_lo1 > big - BN ? big / BN : (core_lo1 + BN - 1) / BN), n_full1 = max(core_hi1 / BN - full1, 0);
+  auto tile_is_full = [&](int tile) -> bool {
+    return ((unsigned)(tile - full0) < (unsigned)n_full0) | ((unsigned)(tile - full1) < (unsigned)n_full1);
+  };
 
-  // MFMA i of S^T = K Q^T: key half i & 1, k-step i >> 1 (the two halves alternate so
-  // that consecutive MFMAs are independent)
+  // The tile loads of an iteration (this wave's share: LPW groups of K, LPW of V) are issued
+  // one at a time between the matrix instructions: as a burst after the barrier they fill the
+  // memory pipeline's queue and the wave sits at its last load until the queue has drained.
+  // They are issued unconditionally, so that the loop has no branches around them: past the
+  // end of the tile list the cursor stays on the last tile, which is then fetched again into
+  // a stage nobody reads any more.
+  constexpr int NL = 2 * KTile::LPW;
+  uint32_t fill_k = 0, fill_v = 0;
+  int64_t fill_k_off = 0, fill_v_off = 0;
+  auto issue_load = [&](int idx) {
+    if (idx < KTile::LPW) KTile::load_group(fill_k, kg + fill_k_off, kv_goff0, p.kv_token_stride, w, idx);
+    else if (idx < NL) VTile::load_group(fill_v, vg + fill_v_off, kv_goff0, p.kv_token_stride, w, idx - KTile::LPW);
+  };
+
+  // Operand i of S^T = K Q^T: key half i & 1, k-step i >> 1 (the two halves alternate so
+  // that consecutive MFMAs are independent); each operand feeds QB MFMAs.
   auto k_operand = [&](const uint16_t* k_lds, int i) { return KTile::read_row(k_lds, k_rd, i & 1, i >> 1); };
 
-  // S^T of tile i on its own.  The range mask enters as the accumulator's initial
+  // S^T of a tile on its own.  The range mask enters as the accumulator's initial
   // value: 0 where the row may look, -inf where it may not.
-  auto multiply_qk = [&](int tile, const uint16_t* k_lds, f32x16 (&s_out)[2]) {
+  auto multiply_qk = [&](int tile, const uint16_t* k_lds, f32x16 (&s_out)[2][QB]) {
     if (wave_sees_all(tile)) {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s_out[nt][e] = 0.0f;
+        for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) s_out[nt][qb][e] = 0.0f;
     } else {
       const int kb = tile * BN + 4 * h;
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          s_out[nt][e] = rng.contains(kb + nt * 32 + 8 * (e / 4) + (e % 4)) ? 0.0f : -INFINITY;
+        for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            s_out[nt][qb][e] = rng[qb].contains(kb + nt * 32 + 8 * (e / 4) + (e % 4)) ? 0.0f : -INFINITY;
     }
     constexpr int N = 2 * KS, AHEAD = 3;
     u32x4 ka[4];
@@ -235,87 +286,107 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
 #pragma unroll
     for (int i2 = 0; i2 < N; ++i2) {
       if (i2 + AHEAD < N) ka[(i2 + AHEAD) & 3] = k_operand(k_lds, i2 + AHEAD);
-      s_out[i2 & 1] = mfma_32x32x16<DTYPE>(ka[i2 & 3], qreg[i2 >> 1], s_out[i2 & 1]);
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+        s_out[i2 & 1][qb] = mfma_32x32x16<DTYPE>(ka[i2 & 3], qreg[qb][i2 >> 1], s_out[i2 & 1][qb]);
+      if ((i2 + 1) % (N / KTile::LPW) == 0) issue_load(i2 / (N / KTile::LPW));
       __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from being hoisted into more registers
     }
   };
 
   // ---- online softmax (log2 domain), in pieces so that it can be interleaved ----
-  u32x4 pb[4];          // P^T of the current tile, packed: the B operand of O^T += V^T P^T
-  float alpha = 1.0f;   // pending rescale of O^T (applied before the tile's P^T is multiplied in)
-  bool rescale = false;
-  float m_use = 0.0f, lsum = 0.0f;
-  auto softmax_max = [&](const f32x16 (&sc)[2]) {
+  u32x4 pb[QB][4];       // P^T of the current tile, packed: the B operands of O^T += V^T P^T
+  float alpha[QB];       // pending rescale of O^T (applied before the tile's P^T is multiplied in)
+  bool rescale[QB];
+  float m_use[QB], lsum[QB];
+  auto softmax_max = [&](const f32x16 (&sc)[2][QB], int qb) {
     float mx = -INFINITY;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[nt][e]);
+      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[nt][qb][e]);
     mx *= p.scale_log2;  // -inf stays -inf (scale > 0)
     mx = fmaxf(mx, xor32(mx));
-    const float m_new = fmaxf(m_run, mx);
-    m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-    rescale = __any(m_new > m_run);
-    alpha = fast_exp2(m_run - m_use);  // m_run = -inf -> 0; 1 where the max did not move
-    l_run *= alpha;
-    m_run = m_new;
-    lsum = 0.0f;
+    // raise the reference maximum only when the tile exceeds it by more than kLazyMax (always
+    // for a row that had none yet: -inf + kLazyMax = -inf), then for every row of the wave
+    rescale[qb] = __any(mx > m_run[qb] + kLazyMax);
+    const float m_new = rescale[qb] ? fmaxf(m_run[qb], mx) : m_run[qb];
+    m_use[qb] = (m_new == -INFINITY) ? 0.0f : m_new;
+    alpha[qb] = fast_exp2(m_run[qb] - m_use[qb]);  // m_run = -inf -> 0; 1 where the maximum stays
+    l_run[qb] *= alpha[qb];
+    m_run[qb] = m_new;
+    lsum[qb] = 0.0f;
   };
-  // elements 2c, 2c+1 of the 32 this lane holds
-  auto softmax_pair = [&](const f32x16 (&sc)[2], int c2) {
+  // elements 2*c2, 2*c2+1 of the 32 this lane holds for query block qb
+  auto softmax_pair = [&](const f32x16 (&sc)[2][QB], int qb, int c2) {
     const int nt = c2 >> 3, e = (c2 & 7) * 2;
-    const float e0 = fast_exp2(fmaf(sc[nt][e], p.scale_log2, -m_use));
-    const float e1 = fast_exp2(fmaf(sc[nt][e + 1], p.scale_log2, -m_use));
-    lsum += e0 + e1;
-    pb[nt * 2 + (e >> 3)][(e & 7) >> 1] = pack2<DTYPE>(e0, e1);
+    const float e0 = fast_exp2(fmaf(sc[nt][qb][e], p.scale_log2, -m_use[qb]));
+    const float e1 = fast_exp2(fmaf(sc[nt][qb][e + 1], p.scale_log2, -m_use[qb]));
+    lsum[qb] += e0 + e1;
+    pb[qb][nt * 2 + (e >> 3)][(e & 7) >> 1] = pack2<DTYPE>(e0, e1);
   };
   auto apply_rescale = [&]() {
-    if (rescale) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+    for (int qb = 0; qb < QB; ++qb)
+      if (rescale[qb]) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
-    }
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o_acc[qb][dt][e] *= alpha[qb];
+      }
   };
-  auto softmax = [&](const f32x16 (&sc)[2]) {
-    softmax_max(sc);
+  auto softmax = [&](const f32x16 (&sc)[2][QB]) {
 #pragma unroll
-    for (int c2 = 0; c2 < 16; ++c2) softmax_pair(sc, c2);
-    l_run += lsum;
+    for (int qb = 0; qb < QB; ++qb) {
+      softmax_max(sc, qb);
+#pragma unroll
+      for (int c2 = 0; c2 < 16; ++c2) softmax_pair(sc, qb, c2);
+      l_run[qb] += lsum[qb];
+    }
   };
 
   // S^T of the next tile and the softmax of the current one in one instruction stream:
   // every MFMA is followed by its share of the softmax arithmetic, so that the matrix
   // pipe and the vector ALU of the SIMD are busy at the same time.  Operands are read
-  // three MFMAs ahead.
-  auto multiply_qk_with_softmax = [&](const uint16_t* k_lds, f32x16 (&s_out)[2], const f32x16 (&sc)[2]) {
-    constexpr int N = 2 * KS;     // MFMAs
+  // three ahead.
+  auto multiply_qk_with_softmax = [&](const uint16_t* k_lds, f32x16 (&s_out)[2][QB], const f32x16 (&sc)[2][QB]) {
+    constexpr int N = 2 * KS;     // operands, QB MFMAs each
     constexpr int AHEAD = 3;
-    constexpr int FIRST = N >= 8 ? 3 : 1;  // MFMAs that carry the max; the pairs follow
+    constexpr int FIRST = N >= 8 ? 3 : 1;  // operands whose MFMAs carry the row maxima; the pairs follow
+    constexpr int PAIRS = 16 * QB;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) s_out[nt][e] = 0.0f;
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_out[nt][qb][e] = 0.0f;
     u32x4 ka[4];
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i) ka[i] = k_operand(k_lds, i);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       if (i + AHEAD < N) ka[(i + AHEAD) & 3] = k_operand(k_lds, i + AHEAD);
-      s_out[i & 1] = mfma_32x32x16<DTYPE>(ka[i & 3], qreg[i >> 1], s_out[i & 1]);
-      if (i == 0) softmax_max(sc);
-      if (i >= FIRST) {
-        const int lo = (i - FIRST) * 16 / (N - FIRST), hi = (i + 1 - FIRST) * 16 / (N - FIRST);
 #pragma unroll
-        for (int c2 = lo; c2 < hi; ++c2) softmax_pair(sc, c2);
+      for (int qb = 0; qb < QB; ++qb) {
+        s_out[i & 1][qb] = mfma_32x32x16<DTYPE>(ka[i & 3], qreg[qb][i >> 1], s_out[i & 1][qb]);
+        if (i == 0) softmax_max(sc, qb);
+        if (i >= FIRST) {
+          // pairs [lo, hi) of the PAIRS this wave owes, query block 0 first
+          const int lo = ((i - FIRST) * QB + qb) * PAIRS / ((N - FIRST) * QB);
+          const int hi = ((i - FIRST) * QB + qb + 1) * PAIRS / ((N - FIRST) * QB);
+#pragma unroll
+          for (int c2 = lo; c2 < hi; ++c2) softmax_pair(sc, c2 / 16, c2 % 16);
+        }
       }
+      if ((i + 1) % (N / KTile::LPW) == 0) issue_load(i / (N / KTile::LPW));
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run += lsum;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) l_run[qb] += lsum[qb];
   };
 
   // O^T += V^T P^T: V^T comes out of the row-major V tile by transpose loads, read
-  // two MFMAs ahead; consecutive MFMAs go to different 32-row tiles of O^T
+  // two operands ahead; consecutive MFMAs go to different accumulators
   auto multiply_pv = [&](const uint16_t* v_lds) {
     constexpr int N = 4 * DT;
     constexpr int AHEAD = 2;
@@ -326,7 +397,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       if (i + AHEAD < N) va[(i + AHEAD) & 3] = v_operand(i + AHEAD);
-      o_acc[i % DT] = mfma_32x32x16<DTYPE>(va[i & 3], pb[i / DT], o_acc[i % DT]);
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+        o_acc[qb][i % DT] = mfma_32x32x16<DTYPE>(va[i & 3], pb[qb][i / DT], o_acc[qb][i % DT]);
+      if ((i + 1) % (N / VTile::LPW) == 0) issue_load(KTile::LPW + i / (N / VTile::LPW));
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -335,26 +409,44 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   // Iteration j multiplies S^T of tile j+1 while it exponentiates tile j, then adds
   // tile j to O^T.  K tile j+1 and V tile j are in LDS by then; K tile j+2 and V tile
   // j+1 stream into the stages that K tile j and V tile j-1 have left.
-  f32x16 s_a[2], s_b[2];
+  f32x16 s_a[2][QB], s_b[2][QB];
   int tile_cur = 0, tile_nxt = 0;  // key tile numbers of list entries j and j+1
   int64_t v_off = 0;               // offset of list entry j+1 (its V is requested in iteration j)
-  auto iteration = [&](int j, f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2], const uint16_t* k_nxt, uint32_t k_fill,
+  bool cur_full = false;           // list entry j lies inside every row's range
+  auto iteration = [&](int j, f32x16 (&s_cur)[2][QB], f32x16 (&s_nxt)[2][QB], const uint16_t* k_nxt, uint32_t k_fill,
                        const uint16_t* v_cur, uint32_t v_fill) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // K tile j+1 and V tile j are filled; nobody reads K tile j or V tile j-1 any more
-    if (j + 2 < n_tiles) KTile::load_async(k_fill, kg + cursor.off, k_goff, w);
-    if (j + 1 < n_tiles) VTile::load_async(v_fill, vg + v_off, v_goff, w);
-    const bool cur = wave_sees(tile_cur), nxt = j + 1 < n_tiles && wave_sees(tile_nxt);
-    if (cur && nxt && wave_sees_all(tile_nxt)) {
+    fill_k = k_fill;
+    fill_v = v_fill;
+    fill_k_off = cursor.off;
+    fill_v_off = v_off;
+    // the S^T product carries the K loads, O^T += V^T P^T the V loads; a wave that skips one
+    // of them still has its share of the tile to request
+    const bool nxt_full = j + 1 < n_tiles && tile_is_full(tile_nxt);
+    bool cur = true;
+    if (cur_full && nxt_full) {
+      // the common case, decided by one test per iteration: this tile and the next are
+      // inside every row's range
       multiply_qk_with_softmax(k_nxt, s_nxt, s_cur);
     } else {
-      if (nxt) multiply_qk(tile_nxt, k_nxt, s_nxt);
+      cur = cur_full || wave_sees(tile_cur);
+      if (j + 1 < n_tiles && (nxt_full || wave_sees(tile_nxt))) {
+        multiply_qk(tile_nxt, k_nxt, s_nxt);
+      } else {
+#pragma unroll
+        for (int i = 0; i < KTile::LPW; ++i) issue_load(i);
+      }
       if (cur) softmax(s_cur);
     }
     if (cur) {
       apply_rescale();
       multiply_pv(v_cur);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VTile::LPW; ++i) issue_load(KTile::LPW + i);
     }
+    cur_full = nxt_full;
     tile_cur = tile_nxt;
     tile_nxt = cursor.tile;
     v_off = cursor.off;
@@ -363,41 +455,52 @@ __global__ __launch_bounds__(kFwdThreads, 2) void attn_fwd_kernel(const AttnFwdP
   if (n_tiles > 0) {
     cursor.seek(runs, 0, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
     tile_cur = cursor.tile;
-    KTile::load_async(k_at0, kg + cursor.off, k_goff, w);
-    VTile::load_async(v_at0, vg + cursor.off, v_goff, w);
+    fill_k = k_at0;
+    fill_v = v_at0;
+    fill_k_off = fill_v_off = cursor.off;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) issue_load(i);
     cursor_next();
     tile_nxt = cursor.tile;
     v_off = cursor.off;
-    if (n_tiles > 1) KTile::load_async(k_at1, kg + cursor.off, k_goff, w);
+    fill_k = k_at1;
+    fill_k_off = cursor.off;
+#pragma unroll
+    for (int i = 0; i < KTile::LPW; ++i) issue_load(i);
     cursor_next();
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    cur_full = tile_is_full(tile_cur);
     if (wave_sees(tile_cur)) multiply_qk(tile_cur, k_lds0, s_a);
     for (int j = 0; j < n_tiles; j += 2) {
       iteration(j, s_a, s_b, k_lds1, k_at0, v_lds0, v_at1);
       if (j + 1 >= n_tiles) break;
       iteration(j + 1, s_b, s_a, k_lds0, k_at1, v_lds1, v_at0);
     }
+    wait_loads();  // the fetches past the end of the list must land before the workgroup's LDS is released
   }
 
   // ---- epilogue ------------------------------------------------------------------
-  const float l_tot = l_run + xor32(l_run);
-  if (!q_valid) return;
-  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   const int o_slot = p.out_block_table[b];
-  uint16_t* op = reinterpret_cast<uint16_t*>(p.out) +
-                 ((int64_t)o_slot * p.block_size + q_local) * q_row_stride + (int64_t)head * D + 4 * h;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int qb = 0; qb < QB; ++qb) {
+    const float l_tot = l_run[qb] + xor32(l_run[qb]);
+    if (!q_valid[qb]) continue;
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    uint16_t* op = reinterpret_cast<uint16_t*>(p.out) +
+                   ((int64_t)o_slot * p.block_size + q_local[qb]) * q_row_stride + (int64_t)head * D + 4 * h;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      u32x2 pk = {pack2<DTYPE>(o_acc[dt][4 * g] * inv, o_acc[dt][4 * g + 1] * inv),
-                  pack2<DTYPE>(o_acc[dt][4 * g + 2] * inv, o_acc[dt][4 * g + 3] * inv)};
-      *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * g) = pk;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 pk = {pack2<DTYPE>(o_acc[qb][dt][4 * g] * inv, o_acc[qb][dt][4 * g + 1] * inv),
+                    pack2<DTYPE>(o_acc[qb][dt][4 * g + 2] * inv, o_acc[qb][dt][4 * g + 3] * inv)};
+        *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * g) = pk;
+      }
+    if (h == 0) {
+      const float lse = l_tot > 0.0f ? (m_run[qb] + log2f(l_tot)) * kLn2 : INFINITY;
+      p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local[qb]] = lse;
     }
-  if (h == 0) {
-    const float lse = l_tot > 0.0f ? (m_run + log2f(l_tot)) * kLn2 : INFINITY;
-    p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local] = lse;
   }
 }
 
@@ -457,7 +560,10 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   p.kv_slot_stride = kv_slot_stride;
   p.kv_token_stride = kv_token_stride;
   p.n_out_slots = n_out_slots;
-  p.q_tiles_per_row = (block_size + kFwdBM - 1) / kFwdBM;
+  // One 32-row query block per wave.  (Two per wave do not pay with this compiler: it cannot
+  // keep the O^T accumulators in the AGPR half of the register file without copies and spills.)
+  const int bm = 128;
+  p.q_tiles_per_row = (block_size + bm - 1) / bm;
   p.scale_log2 = softmax_scale * kLog2e;
   p.n_items = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
   p.xcd_group = p.q_tiles_per_row * (n_heads_q / n_heads_kv);
@@ -466,7 +572,7 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   dim3 grid((unsigned)n_wg), block(kFwdThreads);
   KernelTimer timer("attn_fwd_kernel", stream);
 #define DCP_FWD(DT, HD) \
-  hipLaunchKernelGGL((attn_fwd_kernel<DT, HD>), grid, block, 0, (hipStream_t)stream, p)
+  hipLaunchKernelGGL((attn_fwd_kernel<DT, HD, 1>), grid, block, 0, (hipStream_t)stream, p)
   if (dtype == DCP_DTYPE_BF16) {
     if (head_dim == 128) DCP_FWD(DCP_DTYPE_BF16, 128);
     else DCP_FWD(DCP_DTYPE_BF16, 64);
