@@ -34,6 +34,10 @@ FLAGS = [
     "-target-feature",
     "-Xclang",
     "-packed-fp32-ops",
+    # the attention kernels unroll whole tile streams (48 matrix instructions with their operand
+    # reads and vector work); the default budget for "#pragma unroll" stops short of that
+    "-mllvm",
+    "-pragma-unroll-threshold=262144",
 ]
 
 

@@ -573,6 +573,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
     g_lo1 = min(g_lo1, hull_lds[i][2]);
     g_hi1 = max(g_hi1, hull_lds[i][3]);
   }
+  // the same in every lane: say so, and the tile list, the cursor and the loop control that
+  // derive from them live on the scalar unit
+  g_lo0 = __builtin_amdgcn_readfirstlane(g_lo0);
+  g_hi0 = __builtin_amdgcn_readfirstlane(g_hi0);
+  g_lo1 = __builtin_amdgcn_readfirstlane(g_lo1);
+  g_hi1 = __builtin_amdgcn_readfirstlane(g_hi1);
   const TileRuns runs(g_lo0, g_hi0, g_lo1, g_hi1, BN);
   const int n_tiles = runs.count();
 
