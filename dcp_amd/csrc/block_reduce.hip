@@ -60,7 +60,10 @@ __device__ __forceinline__ bool lse_is_finite(float l) {
 // ---------------------------------------------------------------------------
 constexpr int kMergeThreads = 256;
 
-template <int DTYPE, bool VECTOR>
+// U sources are folded per step and TPG tokens (rows_per_wg apart) are handled by a lane group
+// at once: all their U * TPG 16-byte words and LSEs are requested before any arithmetic, which
+// is what keeps enough bytes in flight when an op has few sources.
+template <int DTYPE, bool VECTOR, int U, int TPG>
 __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
     const typename Elem<DTYPE>::raw* src_out, typename Elem<DTYPE>::raw* dst_out,
     const float* src_lse, float* dst_lse, int n_head, const int32_t* __restrict__ src_block_table,
@@ -72,82 +75,107 @@ __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
   constexpr int VN = VECTOR ? Vec16<DTYPE>::N : 1;
   const int op = blockIdx.x;
   const int n_tok = n_tokens_per_block[op];
+
   // A workgroup takes consecutive tokens of ONE head: its LSE reads and its LSE store are
   // then contiguous floats ([head][token] layout) instead of one 4-byte access per cache
   // line, and every token's head_dim elements are still one contiguous piece.
   const int rows_per_wg = kMergeThreads / lanes_per_row;
   const int h = blockIdx.y % n_head;
-  const int t = (blockIdx.y / n_head) * rows_per_wg + threadIdx.x / lanes_per_row;
+  const int t0 = (blockIdx.y / n_head) * (rows_per_wg * TPG) + threadIdx.x / lanes_per_row;
   const int g = threadIdx.x % lanes_per_row;
-  if (t >= n_tok) return;
+  if (t0 >= n_tok) return;
 
   const int n_src = block_lengths[op];
   const int32_t* table = src_block_table + (int64_t)op * max_n_blocks_per_op;
-  const float* lse_row = src_lse + h * src_lse_head_stride + t * lse_token_stride;
-  const raw* out_row = src_out + t * out_token_stride + (int64_t)h * head_dim;
-  const int64_t dst_tok = (int64_t)dst_token_offsets[op] + t;
+  const float* lse_head = src_lse + h * src_lse_head_stride;
+  const raw* out_head = src_out + (int64_t)h * head_dim;
   const int n_words = head_dim / VN;
+  int t[TPG];
+  bool live[TPG];
+#pragma unroll
+  for (int k = 0; k < TPG; ++k) {
+    live[k] = t0 + k * rows_per_wg < n_tok;
+    t[k] = live[k] ? t0 + k * rows_per_wg : t0;  // a token past the end repeats the first one; never stored
+  }
 
-  // One pass over the sources, four at a time: the four LSEs and the four
-  // 16-byte words are requested before any arithmetic, then folded into a
-  // running (max, sum, weighted out) triple.
-  float row_lse = -1.0f;  // the same in every iteration: it only depends on the LSEs
+  float row_lse[TPG];  // the same in every iteration over w: it only depends on the LSEs
+#pragma unroll
+  for (int k = 0; k < TPG; ++k) row_lse[k] = -1.0f;
   for (int w = g; w < n_words; w += lanes_per_row) {
-    float m = -INFINITY, ssum = 0.0f;
-    float acc[VN];
+    float m[TPG], ssum[TPG], acc[TPG][VN];
 #pragma unroll
-    for (int i = 0; i < VN; ++i) acc[i] = 0.0f;
-    for (int j0 = 0; j0 < n_src; j0 += 4) {
-      float l[4];
-      u32x4 x[4];
-      raw x1[4];
+    for (int k = 0; k < TPG; ++k) {
+      m[k] = -INFINITY;
+      ssum[k] = 0.0f;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int i = 0; i < VN; ++i) acc[k][i] = 0.0f;
+    }
+    for (int j0 = 0; j0 < n_src; j0 += U) {
+      float l[TPG][U];
+      u32x4 x[TPG][U];
+      raw x1[TPG][U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
         const int j = min(j0 + u, n_src - 1);  // tail: re-read the last source, ignored below
         const int64_t blk = table[j];
-        l[u] = lse_row[blk * lse_block_stride];
-        const raw* p = out_row + blk * out_block_stride + (int64_t)w * VN;
-        if constexpr (VECTOR) x[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-        else x1[u] = *p;
+#pragma unroll
+        for (int k = 0; k < TPG; ++k) {
+          l[k][u] = lse_head[t[k] * lse_token_stride + blk * lse_block_stride];
+          const raw* p = out_head + t[k] * out_token_stride + blk * out_block_stride + (int64_t)w * VN;
+          if constexpr (VECTOR) x[k][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+          else x1[k][u] = *p;
+        }
       }
-      float m_new = m;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (j0 + u >= n_src || !lse_is_finite(l[u])) l[u] = -INFINITY;
-        m_new = fmaxf(m_new, l[u]);
+      for (int k = 0; k < TPG; ++k) {
+        float m_new = m[k];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (j0 + u >= n_src || !lse_is_finite(l[k][u])) l[k][u] = -INFINITY;
+          m_new = fmaxf(m_new, l[k][u]);
+        }
+        if (m_new == -INFINITY) continue;  // nothing finite so far
+        const float rescale = expf(m[k] - m_new);  // m = -inf -> 0
+        ssum[k] *= rescale;
+#pragma unroll
+        for (int i = 0; i < VN; ++i) acc[k][i] *= rescale;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const float wgt = expf(l[k][u] - m_new);  // ignored source: exp(-inf) = 0, but its data may be
+          if (l[k][u] == -INFINITY) continue;       // anything, so it is skipped, not multiplied by 0
+          ssum[k] += wgt;
+          if constexpr (VECTOR) fma_vec16<DTYPE>(acc[k], wgt, x[k][u]);
+          else acc[k][0] += wgt * Elem<DTYPE>::load(x1[k][u]);
+        }
+        m[k] = m_new;
       }
-      if (m_new == -INFINITY) continue;  // nothing finite so far
-      const float rescale = expf(m - m_new);  // m = -inf -> 0
-      ssum *= rescale;
+    }
 #pragma unroll
-      for (int i = 0; i < VN; ++i) acc[i] *= rescale;
+    for (int k = 0; k < TPG; ++k) {
+      float new_lse = -1.0f;
+      if (m[k] != -INFINITY) {
+        new_lse = m[k] + logf(ssum[k]);
+        const float inv = 1.0f / ssum[k];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float wgt = expf(l[u] - m_new);  // ignored source: exp(-inf) = 0, but its data may be
-        if (l[u] == -INFINITY) continue;       // anything, so it is skipped, not multiplied by 0
-        ssum += wgt;
-        if constexpr (VECTOR) fma_vec16<DTYPE>(acc, wgt, x[u]);
-        else acc[0] += wgt * Elem<DTYPE>::load(x1[u]);
+        for (int i = 0; i < VN; ++i) acc[k][i] *= inv;
       }
-      m = m_new;
+      row_lse[k] = new_lse;
+      if (!live[k]) continue;
+      const int64_t dst_tok = (int64_t)dst_token_offsets[op] + t[k];
+      raw* q = dst_out + dst_tok * out_token_stride + (int64_t)h * head_dim + (int64_t)w * VN;
+      if constexpr (VECTOR) {
+        __builtin_nontemporal_store(pack_vec16<DTYPE>(acc[k]), reinterpret_cast<u32x4*>(q));
+      } else {
+        *q = Elem<DTYPE>::store(acc[k][0]);
+      }
     }
-    float new_lse = -1.0f;
-    if (m != -INFINITY) {
-      new_lse = m + logf(ssum);
-      const float inv = 1.0f / ssum;
-#pragma unroll
-      for (int i = 0; i < VN; ++i) acc[i] *= inv;
-    }
-    raw* q = dst_out + dst_tok * out_token_stride + (int64_t)h * head_dim + (int64_t)w * VN;
-    if constexpr (VECTOR) {
-      __builtin_nontemporal_store(pack_vec16<DTYPE>(acc), reinterpret_cast<u32x4*>(q));
-    } else {
-      *q = Elem<DTYPE>::store(acc[0]);
-    }
-    row_lse = new_lse;
   }
   // after every read of the sources' LSEs (the destination may be one of them)
-  if (g == 0) dst_lse[h * dst_lse_head_stride + dst_tok * lse_token_stride] = row_lse;
+  if (g == 0) {
+#pragma unroll
+    for (int k = 0; k < TPG; ++k)
+      if (live[k]) dst_lse[h * dst_lse_head_stride + ((int64_t)dst_token_offsets[op] + t[k]) * lse_token_stride] = row_lse[k];
+  }
 }
 
 template <int DTYPE>
@@ -169,7 +197,11 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
   int lpr = 1;
   while (lpr < 64 && n_words % (lpr * 2) == 0) lpr *= 2;
   const int rows_per_wg = kMergeThreads / lpr;
-  const int64_t row_chunks = (int64_t)((block_size + rows_per_wg - 1) / rows_per_wg) * n_head;
+  // sources folded per step x tokens per lane group: eight 16-byte words in flight per lane
+  // (two for a single source, which measured fastest: the op is then a plain copy)
+  const int u = max_n_blocks_per_op >= 4 ? 4 : max_n_blocks_per_op >= 2 ? 2 : 1;
+  const int tpg = u == 4 ? 2 : u == 2 ? 4 : 2;
+  const int64_t row_chunks = (int64_t)((block_size + rows_per_wg * tpg - 1) / (rows_per_wg * tpg)) * n_head;
   DCP_REQUIRE(row_chunks <= 65535, "merge: block of %lld (token, head) rows is too large",
               (long long)block_size * n_head);
   dim3 grid(n_red_ops, (unsigned)row_chunks);
@@ -181,10 +213,15 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
                        out_token_stride, lse_block_stride, lse_token_stride, src_lse_head_stride,
                        dst_lse_head_stride, head_dim, max_n_blocks_per_op, lpr);
   };
-  if (vec)
-    launch(merge_out_lse_kernel<DTYPE, true>);
-  else
-    launch(merge_out_lse_kernel<DTYPE, false>);
+#define DCP_MERGE_PICK(V)                                           \
+  do {                                                              \
+    if (u == 4) launch(merge_out_lse_kernel<DTYPE, V, 4, 2>);       \
+    else if (u == 2) launch(merge_out_lse_kernel<DTYPE, V, 2, 4>);  \
+    else launch(merge_out_lse_kernel<DTYPE, V, 1, 2>);              \
+  } while (0)
+  if (vec) DCP_MERGE_PICK(true);
+  else DCP_MERGE_PICK(false);
+#undef DCP_MERGE_PICK
   return check_launch("merge_out_lse_kernel");
 }
 
@@ -220,18 +257,39 @@ __global__ __launch_bounds__(256) void blockwise_sum_kernel(
   int64_t vec_end = begin;
   if (aligned) {
     vec_end = begin + ((end - begin) / VN) * VN;
+    // kSumUnroll positions x four sources: all their 16-byte words are requested before any
+    // arithmetic (a position past the end repeats the chunk's first word and is not stored)
+    int64_t pos[kSumUnroll];
+    bool live[kSumUnroll];
+    float acc[kSumUnroll][VN];
 #pragma unroll
     for (int u = 0; u < kSumUnroll; ++u) {
       const int64_t i = begin + ((int64_t)u * 256 + threadIdx.x) * VN;
-      if (i >= vec_end) break;
-      float acc[VN];
+      live[u] = i < vec_end;
+      pos[u] = live[u] ? i : begin;
 #pragma unroll
-      for (int k = 0; k < VN; ++k) acc[k] = 0.0f;
-      for (int j = 0; j < n_ops; ++j) {
-        const u32x4 bits = *reinterpret_cast<const u32x4*>(src + offs[j] * src_stride + i);
-        fma_vec16<DTYPE>(acc, 1.0f, bits);
+      for (int k = 0; k < VN; ++k) acc[u][k] = 0.0f;
+    }
+    if (begin < vec_end) {
+      for (int j0 = 0; j0 < n_ops; j0 += 4) {
+        u32x4 bits[4][kSumUnroll];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const raw* row = src + offs[min(j0 + q, n_ops - 1)] * src_stride;  // tail: re-read the last source
+#pragma unroll
+          for (int u = 0; u < kSumUnroll; ++u)
+            bits[q][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + pos[u]));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (j0 + q >= n_ops) break;
+#pragma unroll
+          for (int u = 0; u < kSumUnroll; ++u) fma_vec16<DTYPE>(acc[u], 1.0f, bits[q][u]);
+        }
       }
-      *reinterpret_cast<u32x4*>(dst + i) = pack_vec16<DTYPE>(acc);
+#pragma unroll
+      for (int u = 0; u < kSumUnroll; ++u)
+        if (live[u]) __builtin_nontemporal_store(pack_vec16<DTYPE>(acc[u]), reinterpret_cast<u32x4*>(dst + pos[u]));
     }
   }
   for (int64_t i = vec_end + threadIdx.x; i < end; i += 256) {
