@@ -73,6 +73,33 @@ def workload(name):
             block_size=1024, n_heads=32, n_groups=8, head_dim=128, head_block=4, mask="lambda",
             mask_info=None, mask_kwargs=dict(n_starting=64, l_pretrain=4096),
         )
+    if name == "shared_prefix_96k":
+        # one shared context of 8192 tokens followed by 4..16 independent continuations of
+        # 256..2048 tokens, samples appended until 98304 tokens are filled (the last one is cut)
+        rng = np.random.default_rng(0)
+        seqlens, info, used, total = [], [], 0, 98304
+        while used < total:
+            conts = [int(c) for c in rng.integers(256, 2049, size=int(rng.integers(4, 17)))]
+            room = total - used - 8192
+            if room < 256:  # not even a prefix and one short continuation: lengthen the previous sample
+                seqlens[-1] += total - used
+                info[-1]["continuations"][-1] += total - used
+                break
+            kept = []
+            for c in conts:
+                if room <= 0:
+                    break
+                kept.append(min(c, room))
+                room -= kept[-1]
+            seqlens.append(8192 + sum(kept))
+            info.append(dict(prefix=8192, continuations=kept))
+            used += seqlens[-1]
+        assert sum(seqlens) == total
+        return dict(
+            seqlens=seqlens, block_size=512, n_heads=40, n_groups=8, head_dim=128, head_block=5,
+            mask="shared_prefix", mask_info=info, mask_kwargs={},
+            plan_kwargs=dict(n_kv_groups=2, kv_split="contiguous"),  # every row's kv blocks in two partials: the merge runs
+        )
     if name == "smoke":
         return dict(
             seqlens=[700, 300], block_size=256, n_heads=8, n_groups=2, head_dim=128, head_block=4,
@@ -89,7 +116,7 @@ def build(wl, backward=True):
     mask = MASK_FNS[wl["mask"]](wl["seqlens"], wl["seqlens"], torch.int32, wl["mask_info"], **wl["mask_kwargs"])
     fw, bw, layout = build_single_device_plans(
         wl["seqlens"], wl["block_size"], wl["n_heads"], wl["n_groups"], wl["head_dim"], wl["head_block"],
-        mask, dtype=torch.bfloat16, backward=backward)
+        mask, dtype=torch.bfloat16, backward=backward, **wl.get("plan_kwargs", {}))
     pairs = count_attended_pairs(mask)
     return fw, bw, layout, mask, pairs
 

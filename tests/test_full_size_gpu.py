@@ -4,7 +4,11 @@ and seeded samples of the oracle (the full oracle would take hours):
 * config 2 (Llama-3-8B shape, 65536 tokens, causal, bs 1024, GQA 32/8):
   sampled (sequence, head) parity against dense fp64 attention, exact
   linearity of the backward in dO, bit-reproducibility, HIP-graph replays;
-* config 3 (lambda mask, sink 64 + window 4096) at 32768 tokens: sampled parity;
+* config 3 (lambda mask, sink 64 + window 4096) at 32768 tokens: sampled parity against the
+  oracle; at the full 131072 tokens and config 4 (shared prefix, 98304 tokens, 40/8 heads,
+  bs 512, every row's kv blocks in two partials) a whole (sequence, kv head) group is checked
+  against dense fp64 attention written in plain torch on the GPU (out, LSE, dQ, dK, dV): the
+  numpy oracle would need minutes per sample at these lengths;
 * config 5 (262144 x 32 x 128 bf16 block movement): gather -> inverse scatter is
   the identity bit for bit, padding rows stay untouched, and the 4-way merge is
   invariant under a permutation of its sources.
@@ -70,6 +74,68 @@ def _sample_check(wl, layout, mask, t, samples):
     return worst
 
 
+def _dense_check_gpu(wl, mask, t, s, kvh, chunk=4096):
+    """Dense masked attention of sequence ``s`` for the q heads of kv head ``kvh``, forward and
+    backward, in fp64 with torch matmuls on the GPU, row chunk by row chunk; returns the worst
+    deviations of the kernels' results.  Independent of the kernels under test and of the numpy
+    oracle (whose ``dense_reference`` it restates; both are pinned against each other on a short
+    sequence in ``test_dense_gpu_checker_agrees_with_oracle``)."""
+    from dcp_amd.core.instructions import BufferType as B
+
+    hb, d = wl["head_block"], wl["head_dim"]
+    group = wl["n_heads"] // wl["n_groups"]
+    seq_off = np.concatenate(([0], np.cumsum(wl["seqlens"])))
+    total, L, o0 = int(seq_off[-1]), wl["seqlens"][s], int(seq_off[s])
+    scale = d ** -0.5
+    kv = t[B.LOCAL_KV][kvh * total + o0 : kvh * total + o0 + L].double()  # [L, 2, 1, D]
+    k, v = kv[:, 0, 0], kv[:, 1, 0]
+    m = mask[o0 : o0 + L].to("cuda", torch.int64)
+    if m.dim() == 2:
+        m = torch.stack([m, torch.zeros_like(m)], dim=1)
+    cols = torch.arange(L, device="cuda")[None, :]
+    dk = torch.zeros(L, d, dtype=torch.float64, device="cuda")
+    dv = torch.zeros_like(dk)
+    worst = dict(out=0.0, lse=0.0, dq=0.0, dkv=0.0)
+    rel = lambda g, r: float(((g - r).abs() / r.abs().clamp(min=1.0)).max())
+    hblk, n_hblk = kvh * group // hb, max(1, group // hb)
+    for j in range(n_hblk):
+        sl = slice((hblk + j) * total + o0, (hblk + j) * total + o0 + L)
+        for hh in range(hb):
+            q, do = t[B.LOCAL_Q][sl, hh].double(), t[B.LOCAL_dOUT][sl, hh].double()
+            for r0 in range(0, L, chunk):
+                r1 = min(r0 + chunk, L)
+                mm = m[r0:r1]
+                ok = ((cols >= mm[:, 0, 0:1]) & (cols < mm[:, 0, 1:2])) | ((cols >= mm[:, 1, 0:1]) & (cols < mm[:, 1, 1:2]))
+                sc = (q[r0:r1] @ k.T) * scale
+                sc.masked_fill_(~ok, float("-inf"))
+                lse = torch.logsumexp(sc, dim=1)
+                pr = torch.exp(sc - lse[:, None])
+                out = pr @ v
+                dp = do[r0:r1] @ v.T
+                ds = pr * (dp - (do[r0:r1] * out).sum(1, keepdim=True))
+                dq = (ds @ k) * scale
+                dk += (ds.T @ q[r0:r1]) * scale
+                dv += pr.T @ do[r0:r1]
+                rs = slice(sl.start + r0, sl.start + r1)
+                worst["out"] = max(worst["out"], rel(t[B.LOCAL_OUT][rs, hh].double(), out))
+                worst["lse"] = max(worst["lse"], float((t[B.LOCAL_LSE][hh, rs].double() - lse).abs().max()))
+                worst["dq"] = max(worst["dq"], rel(t[B.LOCAL_dQ][rs, hh].double(), dq))
+    got = t[B.LOCAL_dKV][kvh * total + o0 : kvh * total + o0 + L].double()
+    worst["dkv"] = max(rel(got[:, 0, 0], dk), rel(got[:, 1, 0], dv))
+    return worst
+
+
+def test_dense_gpu_checker_agrees_with_oracle(gpu):
+    """The torch fp64 checker and the numpy oracle see the same deviations on a short sequence."""
+    wl = bench.workload("smoke")
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl, seed=3)
+    a = _sample_check(wl, layout, mask, t, [(0, 1)])
+    b = _dense_check_gpu(wl, mask, t, 0, 1, chunk=256)
+    for key in a:
+        assert abs(a[key] - b[key]) <= 1e-6 + 1e-3 * max(a[key], b[key]), (key, a, b)
+        assert b[key] <= (1e-3 if key == "lse" else 2e-2), b
+
+
 def test_config2_llama_shape_sampled_parity_linearity_determinism(gpu):
     from dcp_amd.core.instructions import BufferType as B
 
@@ -132,6 +198,36 @@ def test_config3_lambda_mask_sampled_parity(gpu):
     samples = [(int(order[-1]) if wl["seqlens"][order[-1]] <= 9000 else int(order[len(order) // 2]), 3)]
     worst = _sample_check(wl, layout, mask, t, samples)
     assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+
+
+def test_config3_lambda_mask_full_size_dense_check(gpu):
+    wl = bench.workload("lambda_128k")
+    assert sum(wl["seqlens"]) == 131072
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl, seed=4)
+    s = int(np.argmax(wl["seqlens"]))  # the longest sequence: most skipped tiles, both ranges in play
+    worst = _dense_check_gpu(wl, mask, t, s, kvh=6)
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+    from dcp_amd.core.instructions import BufferType as B
+    assert bool(torch.isfinite(t[B.LOCAL_LSE]).all()) and bool(torch.isfinite(t[B.LOCAL_dQ].float()).all())
+
+
+def test_config4_shared_prefix_full_size_dense_check(gpu):
+    from dcp_amd.core.instructions import AttnReductionInstr
+
+    wl = bench.workload("shared_prefix_96k")
+    assert sum(wl["seqlens"]) == 98304 and wl["n_heads"] == 40 and wl["head_block"] == 5
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl, seed=5)
+    # the schedule really splits every row's kv blocks over partial outputs: the merge has work to do
+    reds = [i for i in fw.instructions if isinstance(i, AttnReductionInstr)]
+    assert reds and max(len(op.src_buffers) for r in reds for op in r.ops) >= 2
+    s = int(np.argmin(wl["seqlens"]))
+    worst = _dense_check_gpu(wl, mask, t, s, kvh=3)
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+    # closed form of the pair count: p(p+1)/2 + sum_k (c_k p + c_k (c_k+1)/2) per sample
+    from dcp_amd.runtime.flash_attention.utils import count_attended_pairs
+    want = sum(i["prefix"] * (i["prefix"] + 1) // 2 + sum(c * i["prefix"] + c * (c + 1) // 2 for c in i["continuations"])
+               for i in wl["mask_info"])
+    assert count_attended_pairs(mask) == want
 
 
 def test_config5_block_movement_full_size(gpu):
