@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 # cannot be read from inside the benchmark, so the figure is per workload and is only
 # reported for the workload it was measured on.
 MEASURED_TRAFFIC_BYTES = {
-    "llama3_8b_causal_64k": int(((1360743.7 + 1958567.1) * 2.0 + (1302549.4 + 581657.4) * 1.0) * 1024),
+    "llama3_8b_causal_64k": int(((1374594.8 + 2038264.9) * 2.0 + (1302541.6 + 581658.5) * 1.0) * 1024),
 }
 
 
@@ -167,6 +167,40 @@ def time_steps(ex_f, ex_b, fw, bw, steps, warmup):
         step(ex_f, ex_b, fw, bw)
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps
+
+
+def mfma_sustained(iters=60000):
+    """What the matrix cores sustain on this device when a kernel does nothing but bf16
+    32x32x16 MFMAs, one wave per SIMD: with constant operands (full shader clock) and with
+    random N(0,1) operands (the chip lowers its clock under the switching power of real data).
+    The second figure is the practical ceiling the attention kernels can be held against; the
+    roofline `peak` stays the published 2.5 PFLOP/s."""
+    import ctypes
+
+    import torch
+    from dcp_amd import _lib
+
+    n_wg = torch.cuda.get_device_properties(0).multi_processor_count
+    n_words = n_wg * 256 * 16 * 8  # 16 x 16 bytes per thread, as bf16
+    out = torch.empty(2 + n_wg * 256, device="cuda", dtype=torch.float32)
+    res = {}
+    g = torch.Generator(device="cuda").manual_seed(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    for name in ("constant_operands", "random_operands"):
+        ops = (torch.full((n_words,), 0.5, device="cuda") if name == "constant_operands"
+               else torch.randn(n_words, device="cuda", generator=g)).to(torch.bfloat16)
+        flop = ctypes.c_double()
+        args = (ops.data_ptr(), out.data_ptr(), n_wg, iters, 0, ctypes.byref(flop), stream)
+        _lib.call("dcp_mfma_probe", *args)  # warm-up
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.call("dcp_mfma_probe", *args)
+        e1.record()
+        torch.cuda.synchronize()
+        clocks, ticks = out[:2].tolist()
+        res[name] = dict(TFLOPs=round(flop.value / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1),
+                         shader_MHz=round(clocks / ticks * 100.0))
+    return res
 
 
 def kernel_times(ex_f, ex_b, fw, bw, steps):
@@ -345,24 +379,28 @@ def main():
     # The backward is two kernels (dK/dV key-outer, dQ query-outer) that together do
     # the algorithmic backward work 2.5 * fwd; they are priced as one unit.
     dkv, dq, fwd = kt["attn_bwd_dkv_kernel"], kt["attn_bwd_dq_kernel"], kt["attn_fwd_kernel"]
+    # A plan that splits every row's kv blocks over several partials launches each kernel that
+    # many times per step; a launch then does 1/n of the step's work on average.
+    n_launch = max(1, round(dkv["ms_per_step"] / dkv["avg_ms"]))
     bwd_ms = dkv["avg_ms"] + dq["avg_ms"]
-    bwd_tflops = 2.5 * flops_fwd / (bwd_ms * 1e-3) / 1e12
-    fwd_tflops = flops_fwd / (fwd["avg_ms"] * 1e-3) / 1e12
+    bwd_tflops = 2.5 * flops_fwd / n_launch / (bwd_ms * 1e-3) / 1e12
+    fwd_tflops = flops_fwd / n_launch / (fwd["avg_ms"] * 1e-3) / 1e12
     roofline = dict(
         bound="mfma", kernel="attn_bwd_dkv_kernel+attn_bwd_dq_kernel", achieved=round(bwd_tflops, 2),
         peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4),
         traffic=MEASURED_TRAFFIC_BYTES.get(args.workload),
-        flops_per_launch=2.5 * flops_fwd, avg_launch_ms=round(bwd_ms, 4),
+        flops_per_launch=2.5 * flops_fwd / n_launch, avg_launch_ms=round(bwd_ms, 4),
     )
     extra = dict(
         attn_fwd_kernel=dict(achieved_TFLOPs=round(fwd_tflops, 2), frac_of_peak=round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
                              avg_launch_ms=round(fwd["avg_ms"], 4)),
         # executed MFMA work: dK/dV kernel 4 products (S, dP, dV, dK), dQ kernel 3 (S, dP, dQ)
-        attn_bwd_dkv_kernel=dict(executed_TFLOPs=round(2.0 * flops_fwd / (dkv["avg_ms"] * 1e-3) / 1e12, 2),
+        attn_bwd_dkv_kernel=dict(executed_TFLOPs=round(2.0 * flops_fwd / n_launch / (dkv["avg_ms"] * 1e-3) / 1e12, 2),
                                  avg_launch_ms=round(dkv["avg_ms"], 4)),
-        attn_bwd_dq_kernel=dict(executed_TFLOPs=round(1.5 * flops_fwd / (dq["avg_ms"] * 1e-3) / 1e12, 2),
+        attn_bwd_dq_kernel=dict(executed_TFLOPs=round(1.5 * flops_fwd / n_launch / (dq["avg_ms"] * 1e-3) / 1e12, 2),
                                 avg_launch_ms=round(dq["avg_ms"], 4)),
         kernel_ms_per_step={k: round(v["ms_per_step"], 4) for k, v in sorted(kt.items())},
+        mfma_only_kernel=mfma_sustained(),
     )
     if not args.no_movement:
         del ex_f, ex_b

@@ -1,0 +1,73 @@
+// Sustained matrix-core rate of the device, for the roofline discussion: a kernel that does
+// nothing but 32x32x16 MFMAs on operands the caller provides.  What the chip sustains depends
+// on the operand values (power): constant operands run at the full shader clock, random ones
+// do not.  No counterpart in the reference; used by bench.py only.
+#include "attn_common.h"
+
+namespace dcp {
+
+constexpr int kProbeThreads = 256;
+constexpr int kProbeMfmaPerIter = 32;
+
+// One wave per SIMD (launch one workgroup per CU).  Every lane reads 16 operand words
+// (8 A, 8 B) from `operands` and issues kProbeMfmaPerIter MFMAs per iteration on four
+// independent accumulators.  out[0] = shader clocks, out[1] = 100 MHz wall ticks of
+// workgroup 0; out[2 + thread] = a value that depends on every accumulator.
+template <int DTYPE>
+__global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const u32x4* operands, float* out, int iters) {
+  u32x4 a[8], b[8];
+  const size_t base = ((size_t)blockIdx.x * kProbeThreads + threadIdx.x) * 16;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = operands[base + i];
+    b[i] = operands[base + 8 + i];
+  }
+  f32x16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
+  const long long w0 = wall_clock64(), c0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < kProbeMfmaPerIter; ++i) acc[i & 3] = mfma_32x32x16<DTYPE>(a[i & 7], b[(i >> 2) & 7], acc[i & 3]);
+    if ((it & 63) == 63) {  // keep the sums finite
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[j][i] *= 1e-6f;
+    }
+  }
+  const long long c1 = clock64(), w1 = wall_clock64();
+  float r = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) r += acc[j][i];
+  out[2 + (size_t)blockIdx.x * kProbeThreads + threadIdx.x] = r;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    out[0] = (float)(c1 - c0);
+    out[1] = (float)(w1 - w0);
+  }
+}
+
+}  // namespace dcp
+
+using namespace dcp;
+
+extern "C" int dcp_mfma_probe(const void* operands, float* out, int n_workgroups, int iters, int dtype,
+                              double* flop, void* stream) {
+  DCP_REQUIRE(operands && out && flop, "mfma_probe: null argument");
+  DCP_REQUIRE(n_workgroups > 0 && iters > 0, "mfma_probe: sizes must be positive");
+  if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
+    return fail(DCP_ERR_UNSUPPORTED, "mfma_probe: dtype %d unsupported (bf16 and fp16 only)", dtype);
+  *flop = (double)n_workgroups * (kProbeThreads / 64) * (double)iters * kProbeMfmaPerIter * (2.0 * 32 * 32 * 16);
+  dim3 grid(n_workgroups), block(kProbeThreads);
+  if (dtype == DCP_DTYPE_BF16)
+    hipLaunchKernelGGL(mfma_probe_kernel<DCP_DTYPE_BF16>, grid, block, 0, (hipStream_t)stream,
+                       (const u32x4*)operands, out, iters);
+  else
+    hipLaunchKernelGGL(mfma_probe_kernel<DCP_DTYPE_FP16>, grid, block, 0, (hipStream_t)stream,
+                       (const u32x4*)operands, out, iters);
+  return check_launch("mfma_probe_kernel");
+}
