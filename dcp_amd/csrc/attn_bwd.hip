@@ -270,10 +270,13 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
   }
   __syncthreads();
-  const unsigned long long act = mask_lds[0], unm = mask_lds[1];
+  const unsigned long long act = mask_lds[0], unm_v = mask_lds[1];
   const uint32_t act_lo = __builtin_amdgcn_readfirstlane((uint32_t)act);
   const uint32_t act_hi = __builtin_amdgcn_readfirstlane((uint32_t)(act >> 32));
   const unsigned long long act_mask = ((unsigned long long)act_hi << 32) | act_lo;
+  const uint32_t unm_lo = __builtin_amdgcn_readfirstlane((uint32_t)unm_v);
+  const uint32_t unm_hi = __builtin_amdgcn_readfirstlane((uint32_t)(unm_v >> 32));
+  const unsigned long long unm = ((unsigned long long)unm_hi << 32) | unm_lo;
 
   // Everything step (head, qt) reads is requested a step ahead, straight into LDS stage st
   // and with nothing held in registers meanwhile: the Q and dO tiles, and one value per
@@ -291,19 +294,26 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     Tile::load_group(tiles_at + (2 * st + (is_do ? 1 : 0)) * (Tile::SIZE * 2), (is_do ? do_base : q_base) + off, goff0,
                      q_row_stride, w, is_do ? idx - Tile::LPW : idx);
   };
+  // Per-query values of a step, two dword loads per wave and no branches: wave 0 requests the
+  // first range's starts and ends, wave 1 the second range's (the first's again, into planes
+  // nobody reads, when there is one range), wave 2 the LSEs and wave 3 the deltas (each twice,
+  // to the same place).  What depends on the wave's role is fixed here, once.
+  const bool role_rng = w < 2, role_lse = w == 2;
+  const int sc_plane = p.n_ranges == 2 ? 2 * w : 0;
+  const char* sc_base0 = role_rng   ? reinterpret_cast<const char*>(p.attn_range + (int64_t)sc_plane * p.total_q + q_begin)
+                         : role_lse ? reinterpret_cast<const char*>(p.lse + (int64_t)o_slot * p.block_size)
+                                    : reinterpret_cast<const char*>(p.delta + (int64_t)q_begin * p.n_heads_q);
+  const int64_t sc_head_bytes = role_rng ? 0 : role_lse ? (int64_t)p.n_out_slots * p.block_size * 4 : 4;
+  const int64_t sc_second_bytes = role_rng ? (int64_t)p.total_q * 4 : 0;
+  const int sc_query_bytes = (role_rng || role_lse) ? 4 : p.n_heads_q * 4;
+  const uint32_t sc_at0 = role_rng ? rng_at + (2 * w * BM) * 4 : role_lse ? lse_at : delta_at;
+  const uint32_t sc_at_stage = role_rng ? 4 * BM * 4 : BM * 4, sc_at_second = role_rng ? BM * 4 : 0;
   auto request_scalars = [&](int head, int qt, int st) {
     const int ql = min(qt * BM + lane, seqlen_q - 1);
-    if (w < 2) {
-      if (w == 0 || p.n_ranges == 2) {
-        const int32_t* r = p.attn_range + (int64_t)(2 * w) * p.total_q + q_begin + ql;
-        load_async_dword(rng_at + ((st * 4 + 2 * w) * BM) * 4, r);
-        load_async_dword(rng_at + ((st * 4 + 2 * w + 1) * BM) * 4, r + p.total_q);
-      }
-    } else if (w == 2) {
-      load_async_dword(lse_at + st * BM * 4, p.lse + ((int64_t)head * p.n_out_slots + o_slot) * p.block_size + ql);
-    } else {
-      load_async_dword(delta_at + st * BM * 4, p.delta + (int64_t)(q_begin + ql) * p.n_heads_q + head);
-    }
+    const char* base = sc_base0 + head * sc_head_bytes;
+    const uint32_t at = sc_at0 + st * sc_at_stage, voff = (uint32_t)(ql * sc_query_bytes);
+    load_async_dword(at, voff, base);
+    load_async_dword(at + sc_at_second, voff, base + sc_second_bytes);
   };
 
   // steps: (q head of the group) x (active 64-query tile)
@@ -330,8 +340,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed
     // the next step's tiles are requested one load per k-step below: a burst here would
     // hold the wave at its last load until the memory pipeline has taken them all
-    const int head_next = kv_head * group + hg_next, qt_next = __builtin_ctzll(rem);
-    if (more) request_scalars(head_next, qt_next, st ^ 1);
+    // They are issued unconditionally, so that the step has no branches around them: the last
+    // step requests its own tiles once more, into the stage nobody reads any more.
+    const int head_next = more ? kv_head * group + hg_next : kv_head * group + hg;
+    const int qt_next = more ? __builtin_ctzll(rem) : qt;
+    request_scalars(head_next, qt_next, st ^ 1);
     const uint16_t* q_lds = tiles[2 * st];
     const uint16_t* do_lds = tiles[2 * st + 1];
 
@@ -359,23 +372,40 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
-    {
-      // operands are read one k-step ahead of their MFMAs, two k-steps' worth at most live
-      u32x4 aq[2], ad[2];
-      aq[0] = Tile::read_row(q_lds, row_rd, 0, 0);
-      ad[0] = Tile::read_row(do_lds, row_rd, 0, 0);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 1 < KS) {
-          aq[(ks + 1) & 1] = Tile::read_row(q_lds, row_rd, 0, ks + 1);
-          ad[(ks + 1) & 1] = Tile::read_row(do_lds, row_rd, 0, ks + 1);
-        }
-        s_acc = mfma_32x32x16<DTYPE>(aq[ks & 1], kreg[ks], s_acc);
-        if (ks < KS - VL) dp_acc = mfma_32x32x16<DTYPE>(ad[ks & 1], vreg[ks], dp_acc);
-        else dp_acc = mfma_32x32x16<DTYPE>(ad[ks & 1], v_park[w][VL > 0 ? ks - (KS - VL) : 0][lane], dp_acc);
-        if (ks % 2 == 0 && ks / 2 < NL / 2 && more) request_tile(ks / 2, head_next, qt_next, st ^ 1);
-        __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from piling up in registers
+    // Everything the step's 32 MFMAs read from LDS forms one stream, read AHEAD entries ahead
+    // into four rotating registers, across both matrix phases (the first operands of the second
+    // phase are on their way while the vector phase runs):
+    //   phase 1, per k-step: Q rows (-> S), [the parked V k-step (B operand)], dO rows (-> dP)
+    //   phase 2, per (16-query step s2, 32-dim block d): dO^T (-> dV), Q^T (-> dK)
+    constexpr int N1 = 2 * KS + VL, N2 = 4 * DT, NS = N1 + N2, AHEAD = 2;
+    constexpr int FIRST_PARKED = 2 * (KS - VL);  // stream index of the first k-step with a parked V
+    auto entry = [&](int o) -> u32x4 {
+      if (o < N1) {
+        const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
+        const int kind = o < FIRST_PARKED ? (o & 1) * 2 : (o - FIRST_PARKED) % 3;  // 0: Q, 1: parked V, 2: dO
+        if (kind == 1) return v_park[w][VL > 0 ? ks - (KS - VL) : 0][lane];
+        return Tile::read_row(kind == 0 ? q_lds : do_lds, row_rd, 0, ks);
       }
+      const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
+      return Tile::template read_col<true>((i & 1) ? q_lds : do_lds, col_rd, s2, d);
+    };
+    u32x4 buf[4];
+#pragma unroll
+    for (int o = 0; o < AHEAD; ++o) buf[o] = entry(o);
+    int loads_issued = 0;
+    (void)loads_issued;
+#pragma unroll
+    for (int o = 0; o < N1; ++o) {
+      const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
+      const int kind = o < FIRST_PARKED ? (o & 1) * 2 : (o - FIRST_PARKED) % 3;
+      if (kind == 0) s_acc = mfma_32x32x16<DTYPE>(buf[o & 3], kreg[ks], s_acc);
+      else if (kind == 2 && ks < KS - VL) dp_acc = mfma_32x32x16<DTYPE>(buf[o & 3], vreg[ks < KS - VL ? ks : 0], dp_acc);
+      else if (kind == 2) dp_acc = mfma_32x32x16<DTYPE>(buf[o & 3], buf[(o - 1) & 3], dp_acc);
+      // the entry just used (and the one before it) are free: the next read goes there.  Only the
+      // first operand of the second phase is requested before the vector phase (registers)
+      if (o + AHEAD <= N1) buf[(o + AHEAD) & 3] = entry(o + AHEAD);
+      if (kind == 2 && ks % 2 == 0 && ks / 2 < NL / 2) request_tile(ks / 2, head_next, qt_next, st ^ 1);
+      __builtin_amdgcn_sched_barrier(0);  // keeps the order: reads neither pile up in registers nor fall behind
     }
     // ---- P = exp2(S c - lse), dS = P (dP - delta), packed in accumulator order: as B operands
     // they feed the next products without leaving the registers -------------------------------
@@ -396,38 +426,29 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       dsb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(dsv[0], dsv[1]);
       dsb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(dsv[2], dsv[3]);
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int o = N1 + 1; o < N1 + AHEAD; ++o) buf[o & 3] = entry(o);
     // ---- dV^T[dim, key] += dO^T[dim, q] P[q, key];  dK^T[dim, key] += Q^T[dim, q] dS[q, key]
     // over this wave's 32 queries (dO^T and Q^T come out of the row-major tiles by
     // transpose loads, in the accumulators' row order) -----------------------------------------
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-      for (int d2 = 0; d2 < DT; d2 += 2) {
-        u32x4 a_do[2], a_q[2];
-#pragma unroll
-        for (int j = 0; j < 2 && d2 + j < DT; ++j) a_do[j] = Tile::template read_col<true>(do_lds, col_rd, s2, d2 + j);
-#pragma unroll
-        for (int j = 0; j < 2 && d2 + j < DT; ++j) a_q[j] = Tile::template read_col<true>(q_lds, col_rd, s2, d2 + j);
-#pragma unroll
-        for (int j = 0; j < 2 && d2 + j < DT; ++j) {
-          dv_acc[d2 + j] = mfma_32x32x16<DTYPE>(a_do[j], pb[s2], dv_acc[d2 + j]);
-          dk_acc[d2 + j] = mfma_32x32x16<DTYPE>(a_q[j], dsb[s2], dk_acc[d2 + j]);
-        }
-        {
-          constexpr int GROUPS = 2 * ((DT + 1) / 2), PER = (NL / 2 + GROUPS - 1) / GROUPS;
-          const int grp = s2 * ((DT + 1) / 2) + d2 / 2;
-#pragma unroll
-          for (int i = grp * PER; i < (grp + 1) * PER && i < NL / 2; ++i)
-            if (more) request_tile(NL / 2 + i, head_next, qt_next, st ^ 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    for (int o = N1; o < NS; ++o) {
+      const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
+      if (i & 1) dk_acc[d] = mfma_32x32x16<DTYPE>(buf[o & 3], dsb[s2], dk_acc[d]);
+      else dv_acc[d] = mfma_32x32x16<DTYPE>(buf[o & 3], pb[s2], dv_acc[d]);
+      if (o + AHEAD < NS) buf[(o + AHEAD) & 3] = entry(o + AHEAD);
+      constexpr int EVERY = N2 / (NL / 2);  // the second half of the tile loads, evenly over the phase
+      if ((i + 1) % EVERY == 0 && (i + 1) / EVERY <= NL / 2) request_tile(NL / 2 + (i + 1) / EVERY - 1, head_next, qt_next, st ^ 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     st ^= 1;
     hg = hg_next;
   }
 
   // ---- sum the two query halves: the qi = 0 waves finish dV, the qi = 1 waves dK; each
   // wave hands the other product to its partner (same keys) through LDS ----------------------
+  wait_loads();     // the last step's (unused) requests have landed: the tile area is about to be reused
   __syncthreads();  // nobody reads the tiles any more
   float* red = reinterpret_cast<float*>(&tiles[0][0]) + w * (16 * DT * 64);
   {

@@ -114,6 +114,17 @@ __device__ __forceinline__ void load_async_dword(uint32_t lds_at, const void* g)
                : "memory");
 }
 
+// The same with a wave-uniform base address and a per-lane byte offset.
+__device__ __forceinline__ void load_async_dword(uint32_t lds_at, uint32_t lane_offset, const void* base) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  const uint64_t b = ((uint64_t)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_at)), "v"(lane_offset), "s"(b)
+               : "memory");
+}
+
 template <int D, int NW = 4>
 struct KvTile {
   static constexpr int ROWS = 64;
