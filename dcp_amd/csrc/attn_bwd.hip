@@ -611,8 +611,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
 
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
-  uint32_t goff[Tile::LPW];
-  Tile::lane_offsets(goff, p.kv_token_stride, w, lane);
+  const uint32_t kv_goff0 = Tile::lane_offset0(p.kv_token_stride, w, lane);
   const int row_rd = Tile::row_base(c, h);
   const int col_rd = Tile::col_base(lane, true);
 
@@ -620,9 +619,17 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   const int tiles_per_block = p.block_size / BN;
   const int64_t tile_stride = (int64_t)BN * p.kv_token_stride;
   TileCursor cursor;
-  auto fetch = [&](uint32_t k_dst, uint32_t v_dst) {
-    Tile::load_async(k_dst, kg + cursor.off, goff, w);
-    Tile::load_async(v_dst, vg + cursor.off, goff, w);
+  // This wave's share of a tile's loads (LPW groups of K, then LPW of V) is issued one load at a
+  // time between the matrix instructions, and unconditionally, so that no branch surrounds a
+  // load: past the end of the list the cursor stays on the last tile, which is then fetched
+  // again into a stage nobody reads any more.
+  constexpr int NL = 2 * Tile::LPW;
+  uint32_t fill_k = 0, fill_v = 0;
+  auto issue_load = [&](int idx) {
+    if (idx < Tile::LPW) Tile::load_group(fill_k, kg + cursor.off, kv_goff0, p.kv_token_stride, w, idx);
+    else if (idx < NL) Tile::load_group(fill_v, vg + cursor.off, kv_goff0, p.kv_token_stride, w, idx - Tile::LPW);
+  };
+  auto advance = [&]() {
     if (cursor.index + 1 < n_tiles)
       cursor.advance(runs, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
   };
@@ -630,7 +637,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   auto compute = [&](int kt, const uint16_t* k_lds, const uint16_t* v_lds) {
     const int k0 = kt * BN;
     const bool wave_active = (k0 < w_hi0 && k0 + BN > w_lo0) || (k0 < w_hi1 && k0 + BN > w_lo1);
-    if (!wave_active) return;
+    if (!wave_active) {  // its share of the next tile is still to be requested
+#pragma unroll
+      for (int i = 0; i < NL; ++i) issue_load(i);
+      return;
+    }
     const bool unmasked = (core_lo0 <= k0 && k0 + BN <= core_hi0) || (core_lo1 <= k0 && k0 + BN <= core_hi1);
 
     u32x4 dsb[4];
@@ -661,6 +672,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
           s_acc = mfma_32x32x16<DTYPE>(ka[k4], qreg[half * 4 + k4], s_acc);
           dp_acc = mfma_32x32x16<DTYPE>(va[k4], doreg[half * 4 + k4], dp_acc);
         }
+        // one tile load per group of eight MFMAs: 2 * KS / 4 of the NL here, the rest below
+        if (nt * (KS / 4) + half < NL / 2) issue_load(nt * (KS / 4) + half);
       }
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
@@ -688,26 +701,38 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
       }
 #pragma unroll
       for (int s2 = 0; s2 < 4; ++s2) dq_acc[dt] = mfma_32x32x16<DTYPE>(kt_a[dt & 1][s2], dsb[s2], dq_acc[dt]);
+      if (NL / 2 + dt < NL) issue_load(NL / 2 + dt);
     }
+#pragma unroll
+    for (int i = NL / 2 + DT; i < NL; ++i) issue_load(i);
   };
 
   const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
   const uint32_t v_at0 = lds_address(v_lds0), v_at1 = lds_address(v_lds1);
   if (n_tiles > 0) {
     cursor.seek(runs, 0, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
-    fetch(k_at0, v_at0);
+    fill_k = k_at0;
+    fill_v = v_at0;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) issue_load(i);
+    advance();
   }
   for (int i = 0; i < n_tiles; i += 2) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
-    if (i + 1 < n_tiles) fetch(k_at1, v_at1);
-    compute(runs.tile(i), k_lds0, v_lds0);
+    fill_k = k_at1;
+    fill_v = v_at1;
+    compute(runs.tile(i), k_lds0, v_lds0);  // requests list entry i + 1 (or the last tile again)
+    advance();
     if (i + 1 >= n_tiles) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
-    if (i + 2 < n_tiles) fetch(k_at0, v_at0);
+    fill_k = k_at0;
+    fill_v = v_at0;
     compute(runs.tile(i + 1), k_lds1, v_lds1);
+    advance();
   }
+  if (n_tiles > 0) wait_loads();  // the fetch past the end of the list must land before the LDS is released
 
   if (!q_valid) return;
   uint16_t* op = reinterpret_cast<uint16_t*>(p.dq) +
