@@ -357,17 +357,24 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 #pragma unroll
       for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
     } else {
+      // the four queries of an accumulator register group are consecutive: their range planes
+      // come in 16-byte reads, requested together before the comparisons.  With one range the
+      // second range's planes hold the first's again (see request_scalars): the union is the same.
+      typedef int i32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = qi * 32 + acc_row(i, h);
-        const int s0 = rng_lds[st][0][r], len0 = min(rng_lds[st][1][r], seqlen_kv) - s0;
-        bool ok = (unsigned)(kv - s0) < (unsigned)max(len0, 0);
-        if (p.n_ranges == 2) {
-          const int s1 = rng_lds[st][2][r], len1 = min(rng_lds[st][3][r], seqlen_kv) - s1;
-          ok |= (unsigned)(kv - s1) < (unsigned)max(len1, 0);
+      for (int g = 0; g < 4; ++g) {
+        i32x4 rs[4];
+#pragma unroll
+        for (int pl = 0; pl < 4; ++pl) rs[pl] = *reinterpret_cast<const i32x4*>(&rng_lds[st][pl][qi * 32 + 8 * g + 4 * h]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int s0 = rs[0][r], len0 = min(rs[1][r], seqlen_kv) - s0;
+          const int s1 = rs[2][r], len1 = min(rs[3][r], seqlen_kv) - s1;
+          bool ok = ((unsigned)(kv - s0) < (unsigned)max(len0, 0)) | ((unsigned)(kv - s1) < (unsigned)max(len1, 0));
+          ok &= qt * BM + qi * 32 + 8 * g + 4 * h + r < seqlen_q;
+          s_acc[4 * g + r] = ok ? 0.0f : -INFINITY;
         }
-        ok &= qt * BM + r < seqlen_q;
-        s_acc[i] = ok ? 0.0f : -INFINITY;
+        __builtin_amdgcn_sched_barrier(0);  // one group's planes in registers at a time
       }
     }
 #pragma unroll
