@@ -696,22 +696,23 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
         dsb[nt * 2 + g] = packed;
       }
     }
-    // dQ^T[d, q] += K^T[d, kv] dS^T[kv, q]: K^T comes out of the K tile by transpose loads
-    u32x4 kt_a[2][4];
+    // dQ^T[d, q] += K^T[d, kv] dS^T[kv, q]: K^T comes out of the K tile by transpose loads, one
+    // 16-key step ahead; consecutive MFMAs go to different accumulators
+    u32x4 kt_a[2][DT];
 #pragma unroll
-    for (int s2 = 0; s2 < 4; ++s2) kt_a[0][s2] = Tile::template read_col<true>(k_lds, col_rd, s2, 0);
+    for (int dt = 0; dt < DT; ++dt) kt_a[0][dt] = Tile::template read_col<true>(k_lds, col_rd, 0, dt);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      if (dt + 1 < DT) {
+    for (int s2 = 0; s2 < 4; ++s2) {
+      if (s2 + 1 < 4) {
 #pragma unroll
-        for (int s2 = 0; s2 < 4; ++s2) kt_a[(dt + 1) & 1][s2] = Tile::template read_col<true>(k_lds, col_rd, s2, dt + 1);
+        for (int dt = 0; dt < DT; ++dt) kt_a[(s2 + 1) & 1][dt] = Tile::template read_col<true>(k_lds, col_rd, s2 + 1, dt);
       }
 #pragma unroll
-      for (int s2 = 0; s2 < 4; ++s2) dq_acc[dt] = mfma_32x32x16<DTYPE>(kt_a[dt & 1][s2], dsb[s2], dq_acc[dt]);
-      if (NL / 2 + dt < NL) issue_load(NL / 2 + dt);
+      for (int dt = 0; dt < DT; ++dt) dq_acc[dt] = mfma_32x32x16<DTYPE>(kt_a[s2 & 1][dt], dsb[s2], dq_acc[dt]);
+      if (NL / 2 + s2 < NL) issue_load(NL / 2 + s2);
     }
 #pragma unroll
-    for (int i = NL / 2 + DT; i < NL; ++i) issue_load(i);
+    for (int i = NL / 2 + 4; i < NL; ++i) issue_load(i);
   };
 
   const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
