@@ -276,6 +276,22 @@ def movement_microbench(iters=5, bs=512):
     n, total = _lib.profile_report()["merge_out_lse_kernel"]
     merge_bytes = (n_src + 1) * (d * 2 + 4) * tokens * heads
     merge_gbps = merge_bytes / (total / n * 1e-3) / 1e9
+
+    # what a plain streaming kernel reaches at the same read : write mixes on the same buffers
+    # (1 read + 1 write like the copy, 4 reads + 1 write like the merge): the practical ceiling
+    stream_gbps = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    per_stream = tokens * heads * d * 2  # 2 GiB
+    for ns in (1, 4):
+        call = lambda: _lib.call("dcp_hbm_stream_probe", outs.data_ptr(), dst_out.data_ptr(), ns, per_stream, stream)
+        call()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        stream_gbps[ns] = (ns + 1) * per_stream / (e0.elapsed_time(e1) / iters * 1e-3) / 1e9
     return dict(
         workload="block movement: 262144 tok x 32 heads x 128 bf16, 512-token blocks, seeded permutation",
         gather_scatter_GBps=round(copy_gbps, 1),
@@ -285,6 +301,8 @@ def movement_microbench(iters=5, bs=512):
         merge4_GBps=round(merge_gbps, 1),
         merge4_frac_of_8TBps=round(merge_gbps / PEAK_HBM_GBPS, 4),
         merge_bytes_per_launch=merge_bytes,
+        plain_stream_1r1w_GBps=round(stream_gbps[1], 1),
+        plain_stream_4r1w_GBps=round(stream_gbps[4], 1),
     )
 
 

@@ -1,4 +1,7 @@
-// Sustained matrix-core rate of the device, for the roofline discussion: a kernel that does
+// Two probes for the roofline discussion (no counterpart in the reference; used by bench.py
+// only): the sustained matrix-core rate and the streaming rate of HBM.
+//
+// Sustained matrix-core rate of the device: a kernel that does
 // nothing but 32x32x16 MFMAs on operands the caller provides.  What the chip sustains depends
 // on the operand values (power): constant operands run at the full shader clock, random ones
 // do not.  No counterpart in the reference; used by bench.py only.
@@ -51,9 +54,56 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const u32x
   }
 }
 
+// Plain streaming kernel for the HBM roofline discussion: NS equally long input streams are
+// added 16 bytes at a time (non-temporal loads) and written once (non-temporal store).  What
+// this reaches is the practical ceiling for the gather / merge / sum kernels at the same
+// read : write mix.
+template <int NS>
+__global__ __launch_bounds__(256) void hbm_stream_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                         size_t words_per_stream) {
+  constexpr int UNR = 2;
+  const size_t base = (size_t)blockIdx.x * 256 * UNR + threadIdx.x;
+  u32x4 v[NS][UNR];
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) v[s][u] = __builtin_nontemporal_load(src + s * words_per_stream + base + u * 256);
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    u32x4 acc = v[0][u];
+#pragma unroll
+    for (int s = 1; s < NS; ++s) acc += v[s][u];
+    __builtin_nontemporal_store(acc, dst + base + u * 256);
+  }
+}
+
 }  // namespace dcp
 
 using namespace dcp;
+
+extern "C" int dcp_hbm_stream_probe(const void* src, void* dst, int n_streams, size_t bytes_per_stream,
+                                    void* stream) {
+  DCP_REQUIRE(src && dst, "hbm_stream_probe: null argument");
+  DCP_REQUIRE(bytes_per_stream > 0 && bytes_per_stream % (256 * 2 * 16) == 0,
+              "hbm_stream_probe: bytes_per_stream must be a positive multiple of 8192");
+  DCP_REQUIRE(bytes_per_stream / 8192 < ((size_t)1 << 31), "hbm_stream_probe: stream too long");
+  const size_t words = bytes_per_stream / 16;
+  dim3 grid((unsigned)(bytes_per_stream / 8192)), block(256);
+  switch (n_streams) {
+    case 1:
+      hipLaunchKernelGGL(hbm_stream_kernel<1>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words);
+      break;
+    case 2:
+      hipLaunchKernelGGL(hbm_stream_kernel<2>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words);
+      break;
+    case 4:
+      hipLaunchKernelGGL(hbm_stream_kernel<4>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words);
+      break;
+    default:
+      return fail(DCP_ERR_UNSUPPORTED, "hbm_stream_probe: n_streams %d unsupported (1, 2 or 4)", n_streams);
+  }
+  return check_launch("hbm_stream_kernel");
+}
 
 extern "C" int dcp_mfma_probe(const void* operands, float* out, int n_workgroups, int iters, int dtype,
                               double* flop, void* stream) {

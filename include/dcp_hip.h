@@ -69,6 +69,16 @@ int dcp_mfma_probe(const void* operands, float* out, int n_workgroups, int iters
                    double* flop, void* stream);
 
 /*
+ * Streaming rate of HBM, for the roofline discussion (no counterpart in the
+ * reference; used by the benchmark only).  Adds `n_streams` (1, 2 or 4) equally
+ * long input streams, laid end to end in `src`, 16 bytes at a time and writes
+ * the sum to `dst`: n_streams reads and one write of `bytes_per_stream` (a
+ * multiple of 8192) each.  Time it with events on `stream`.
+ */
+int dcp_hbm_stream_probe(const void* src, void* dst, int n_streams, size_t bytes_per_stream,
+                         void* stream);
+
+/*
  * Block gather / scatter through pointer tables.
  * Replaces dcp.ops.fused_ops.fused_copy_{bf16,fp16,fp32}_varlen
  * (dcp/ops/fused_ops.py:842-864, 916-938, 1013-1035; kernels :290-335,
