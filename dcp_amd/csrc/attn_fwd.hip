@@ -33,8 +33,6 @@
 // the per-element range test.
 #include <math.h>
 
-#include <algorithm>
-
 #include "attn_common.h"
 
 namespace dcp {
@@ -85,9 +83,8 @@ constexpr float kLazyMax = 8.0f;
 // K / V^T operand read from LDS feeds two matrix instructions and every tile brought into LDS
 // serves twice the arithmetic; the wave then needs the whole register file (one workgroup
 // per CU, accumulators in the AGPR half).
-// One work item: `item` names a (row, head, query tile).
 template <int DTYPE, int D, int QB>
-__device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) {
+__global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
   constexpr int BN = kFwdBN;
   constexpr int BM = 128 * QB;
   constexpr int KS = D / 16;  // k-steps of S^T = K Q^T
@@ -110,7 +107,9 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
   const int h = lane >> 5;
 
   // ---- which (row, head, q tile) ----------------------------------------
-  int wg = item;
+  // the query tiles and grouped heads of a row share its K/V: keep them on one XCD
+  int wg = xcd_logical_id(blockIdx.x, p.xcd_group, p.n_items);
+  if (wg < 0) return;
   const int qt = wg % p.q_tiles_per_row;
   wg /= p.q_tiles_per_row;
   const int head = wg % p.n_heads_q;
@@ -518,30 +517,6 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
   }
 }
 
-// The kernel is persistent: the launch has (at most) as many workgroups as the device holds at
-// once, and each walks a fixed share of the work items.  A grid of one workgroup per item loses
-// a tenth of the device to dispatch: workgroup ids are dealt to the 8 XCDs strictly in turn, so
-// an XCD with a free slot waits until every XCD before it in the turn has taken its workgroup
-// (13 us between two workgroups of a CU slot on average, against 100 us of work).
-//
-// Workgroup b sits on XCD b % 8 and is the (b / 8)-th of its XCD's L workgroups.  The items that
-// stream the same K/V (the query tiles and grouped heads of a row, `xcd_group` of them with
-// consecutive ids) stay on one XCD: stream s belongs to XCD s % 8.  The rows come longest first,
-// so an XCD's item list is in descending order of work, and its workgroups take it in serpentine
-// rounds (0..L-1, L-1..0, ...), which evens out their sums without any counter.
-template <int DTYPE, int D, int QB>
-__global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
-  const int x = blockIdx.x % kNumXcd, l = blockIdx.x / kNumXcd, n_l = gridDim.x / kNumXcd;
-  const int64_t n_streams = (p.n_items + p.xcd_group - 1) / p.xcd_group;
-  const int64_t n_x = n_streams > x ? (n_streams - x + kNumXcd - 1) / kNumXcd * p.xcd_group : 0;  // items of this XCD
-  for (int64_t round = 0; round * n_l < n_x; ++round) {
-    const int64_t i = round * n_l + ((round & 1) ? n_l - 1 - l : l);
-    const int64_t item = (x + kNumXcd * (i / p.xcd_group)) * p.xcd_group + i % p.xcd_group;
-    if (i < n_x && item < p.n_items) attn_fwd_item<DTYPE, D, QB>(p, (int)item);
-    __syncthreads();  // the next item reuses the LDS tables and tiles
-  }
-}
-
 }  // namespace dcp
 
 using namespace dcp;
@@ -605,9 +580,8 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   p.scale_log2 = softmax_scale * kLog2e;
   p.n_items = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
   p.xcd_group = p.q_tiles_per_row * (n_heads_q / n_heads_kv);
-  DCP_REQUIRE(p.n_items < ((int64_t)1 << 31), "attn_fwd: too many work items");
-  // as many workgroups as the device holds at once (two per CU), a multiple of the XCD count
-  const int64_t n_wg = std::min<int64_t>(xcd_grid_size(p.n_items, 1), 2 * (int64_t)device_cu_count());
+  const int64_t n_wg = xcd_grid_size(p.n_items, p.xcd_group);
+  DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_fwd: grid too large");
   dim3 grid((unsigned)n_wg), block(kFwdThreads);
   KernelTimer timer("attn_fwd_kernel", stream);
 #define DCP_FWD(DT, HD) \
