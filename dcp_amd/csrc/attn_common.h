@@ -46,7 +46,24 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 // below 2^-126 flush to zero, which is what a softmax weight that small is).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
+// The value the other half of the wave holds (lane ^ 32), by one register swap on the vector
+// unit (no trip through LDS).
+__device__ __forceinline__ float xor32(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // {lanes 0-31 twice, lanes 32-63 twice}
+  return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+}
+// max / sum over the two halves, the same in both
+__device__ __forceinline__ float halves_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 __device__ __forceinline__ int wave_min(int x) {
 #pragma unroll

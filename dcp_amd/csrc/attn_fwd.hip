@@ -309,14 +309,21 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   float alpha[QB];       // pending rescale of O^T (applied before the tile's P^T is multiplied in)
   bool rescale[QB];
   float m_use[QB], lsum[QB];
-  auto softmax_max = [&](const f32x16 (&sc)[2][QB], int qb) {
-    float mx = -INFINITY;
+  // The row maximum of a tile is taken in kMaxParts pieces of 32 / kMaxParts elements and
+  // a final step, so that it can be spread between matrix instructions.
+  constexpr int kMaxParts = 4;
+  float mx_part[QB];
+  auto row_max_part = [&](const f32x16 (&sc)[2][QB], int qb, int part) {
+    constexpr int PER = 32 / kMaxParts;
+    float mx = part == 0 ? -INFINITY : mx_part[qb];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[nt][qb][e]);
-    mx *= p.scale_log2;  // -inf stays -inf (scale > 0)
-    mx = fmaxf(mx, xor32(mx));
+    for (int i = 0; i < PER; ++i) mx = fmaxf(mx, sc[(part * PER + i) >> 4][qb][(part * PER + i) & 15]);
+    mx_part[qb] = mx;
+  };
+  // `valid` false (the accumulators hold no tile): as if every element were masked, nothing changes
+  auto row_max_finish = [&](int qb, bool valid) {
+    float mx = valid ? mx_part[qb] * p.scale_log2 : -INFINITY;  // -inf stays -inf (scale > 0)
+    mx = halves_max(mx);
     // raise the reference maximum only when the tile exceeds it by more than kLazyMax (always
     // for a row that had none yet: -inf + kLazyMax = -inf), then for every row of the wave
     rescale[qb] = __any(mx > m_run[qb] + kLazyMax);
@@ -326,6 +333,16 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     l_run[qb] *= alpha[qb];
     m_run[qb] = m_new;
     lsum[qb] = 0.0f;
+  };
+  // The maximum step of tile j+1 runs at the end of iteration j (inside O^T += V^T P^T of tile j
+  // on the fast path), off the head of the exponentials' dependency chain.
+  auto softmax_max = [&](const f32x16 (&sc)[2][QB]) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+#pragma unroll
+      for (int part = 0; part < kMaxParts; ++part) row_max_part(sc, qb, part);
+      row_max_finish(qb, true);
+    }
   };
   // elements 2*c2, 2*c2+1 of the 32 this lane holds for query block qb
   auto softmax_pair = [&](const f32x16 (&sc)[2][QB], int qb, int c2) {
@@ -348,7 +365,6 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   auto softmax = [&](const f32x16 (&sc)[2][QB]) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      softmax_max(sc, qb);
 #pragma unroll
       for (int c2 = 0; c2 < 16; ++c2) softmax_pair(sc, qb, c2);
       l_run[qb] += lsum[qb];
@@ -362,7 +378,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   auto multiply_qk_with_softmax = [&](const uint16_t* k_lds, f32x16 (&s_out)[2][QB], const f32x16 (&sc)[2][QB]) {
     constexpr int N = 2 * KS;     // operands, QB MFMAs each
     constexpr int AHEAD = 3;
-    constexpr int FIRST = N >= 8 ? 3 : 1;  // operands whose MFMAs carry the row maxima; the pairs follow
+    constexpr int FIRST = 0;
     constexpr int PAIRS = 16 * QB;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
@@ -379,7 +395,6 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         s_out[i & 1][qb] = mfma_32x32x16<DTYPE>(ka[i & 3], qreg[qb][i >> 1], s_out[i & 1][qb]);
-        if (i == 0) softmax_max(sc, qb);
         if (i >= FIRST) {
           // pairs [lo, hi) of the PAIRS this wave owes, query block 0 first
           const int lo = ((i - FIRST) * QB + qb) * PAIRS / ((N - FIRST) * QB);
@@ -396,8 +411,9 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   };
 
   // O^T += V^T P^T: V^T comes out of the row-major V tile by transpose loads, read
-  // two operands ahead; consecutive MFMAs go to different accumulators
-  auto multiply_pv = [&](const uint16_t* v_lds) {
+  // two operands ahead; consecutive MFMAs go to different accumulators.  The row maxima of the
+  // next tile (S^T in s_next if has_next) are taken between the first MFMAs.
+  auto multiply_pv = [&](const uint16_t* v_lds, const f32x16 (&s_next)[2][QB], bool has_next) {
     constexpr int N = 4 * DT;
     constexpr int AHEAD = 2;
     auto v_operand = [&](int i) { return VTile::template read_col<true>(v_lds, v_rd, i / DT, i % DT); };
@@ -410,6 +426,17 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
         o_acc[qb][i % DT] = mfma_32x32x16<DTYPE>(va[i & 3], pb[qb][i / DT], o_acc[qb][i % DT]);
+      {
+        // a piece after every second MFMA
+        constexpr int STEP = N >= 2 * (kMaxParts + 1) ? 2 : 1;
+        if (i % STEP == STEP - 1 && i / STEP <= kMaxParts) {
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            if (i / STEP < kMaxParts) row_max_part(s_next, qb, i / STEP);
+            else row_max_finish(qb, has_next);
+          }
+        }
+      }
       if ((i + 1) % (N / VTile::LPW) == 0) issue_load(KTile::LPW + i / (N / VTile::LPW));
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -420,6 +447,12 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   // tile j to O^T.  K tile j+1 and V tile j are in LDS by then; K tile j+2 and V tile
   // j+1 stream into the stages that K tile j and V tile j-1 have left.
   f32x16 s_a[2][QB], s_b[2][QB];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s_a[nt][qb][e] = s_b[nt][qb][e] = 0.0f;
   int tile_cur = 0, tile_nxt = 0;  // key tile numbers of list entries j and j+1
   int64_t v_off = 0;               // offset of list entry j+1 (its V is requested in iteration j)
   bool cur_full = false;           // list entry j lies inside every row's range
@@ -434,7 +467,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     // the S^T product carries the K loads, O^T += V^T P^T the V loads; a wave that skips one
     // of them still has its share of the tile to request
     const bool nxt_full = j + 1 < n_tiles && tile_is_full(tile_nxt);
-    bool cur = true;
+    bool cur = true, nxt = true;
     if (cur_full && nxt_full) {
       // the common case, decided by one test per iteration: this tile and the next are
       // inside every row's range
@@ -442,7 +475,8 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
       multiply_qk_with_softmax(k_nxt, s_nxt, s_cur);
     } else {
       cur = cur_full || wave_sees(tile_cur);
-      if (j + 1 < n_tiles && (nxt_full || wave_sees(tile_nxt))) {
+      nxt = j + 1 < n_tiles && (nxt_full || wave_sees(tile_nxt));
+      if (nxt) {
         multiply_qk(tile_nxt, k_nxt, s_nxt);
       } else {
 #pragma unroll
@@ -453,11 +487,12 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     if (cur) {
       apply_rescale();
       __builtin_amdgcn_s_setprio(kPrioDense);
-      multiply_pv(v_cur);
+      multiply_pv(v_cur, s_nxt, nxt);
       __builtin_amdgcn_s_setprio(kPrioControl);
     } else {
 #pragma unroll
       for (int i = 0; i < VTile::LPW; ++i) issue_load(KTile::LPW + i);
+      if (nxt) softmax_max(s_nxt);
     }
     cur_full = nxt_full;
     tile_cur = tile_nxt;
@@ -484,7 +519,10 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     cur_full = tile_is_full(tile_cur);
-    if (wave_sees(tile_cur)) multiply_qk(tile_cur, k_lds0, s_a);
+    if (wave_sees(tile_cur)) {
+      multiply_qk(tile_cur, k_lds0, s_a);
+      softmax_max(s_a);
+    }
     for (int j = 0; j < n_tiles; j += 2) {
       iteration(j, s_a, s_b, k_lds1, k_at0, v_lds0, v_at1);
       if (j + 1 >= n_tiles) break;
@@ -497,7 +535,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   const int o_slot = p.out_block_table[b];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const float l_tot = l_run[qb] + xor32(l_run[qb]);
+    const float l_tot = halves_sum(l_run[qb]);
     if (!q_valid[qb]) continue;
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     uint16_t* op = reinterpret_cast<uint16_t*>(p.out) +
