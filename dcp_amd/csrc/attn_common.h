@@ -350,7 +350,7 @@ struct TileCursor {
   // to the next tile of the list (call only while index + 1 < runs.count())
   __device__ __forceinline__ void advance(const TileRuns& runs, int tiles_per_block, const int* slot_lds,
                                           const int32_t* kv_table, int64_t slot_stride, int64_t tile_stride) {
-    if (index + 1 == runs.b0 - runs.a0) {  // jump to the second run
+    if (__builtin_expect(index + 1 == runs.b0 - runs.a0, 0)) {  // jump to the second run
       seek(runs, index + 1, tiles_per_block, slot_lds, kv_table, slot_stride, tile_stride);
       return;
     }
@@ -358,7 +358,7 @@ struct TileCursor {
     ++tile;
     ++pos;
     off += tile_stride;
-    if (pos == tiles_per_block) {
+    if (__builtin_expect(pos == tiles_per_block, 0)) {
       pos = 0;
       ++blk;
       off = (int64_t)slot(slot_lds, kv_table, blk) * slot_stride;

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   const int64_t tile_stride = (int64_t)BN * p.kv_token_stride;
   TileCursor cursor;
   auto cursor_next = [&]() {
-    if (cursor.index + 1 < n_tiles) cursor.advance(runs, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
+    if (__builtin_expect(cursor.index + 1 < n_tiles, 1)) cursor.advance(runs, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
     else ++cursor.index;  // past the end: nothing left to request
   };
   const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   auto apply_rescale = [&]() {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
-      if (rescale[qb]) {
+      if (__builtin_expect(rescale[qb], 0)) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     // of them still has its share of the tile to request
     const bool nxt_full = j + 1 < n_tiles && tile_is_full(tile_nxt);
     bool cur = true, nxt = true;
-    if (cur_full && nxt_full) {
+    if (__builtin_expect(cur_full && nxt_full, 1)) {
       // the common case, decided by one test per iteration: this tile and the next are
       // inside every row's range
       __builtin_amdgcn_s_setprio(kPrioFused);
@@ -484,7 +484,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
       }
       if (cur) softmax(s_cur);
     }
-    if (cur) {
+    if (__builtin_expect(cur, 1)) {
       apply_rescale();
       __builtin_amdgcn_s_setprio(kPrioDense);
       multiply_pv(v_cur, s_nxt, nxt);
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     }
     for (int j = 0; j < n_tiles; j += 2) {
       iteration(j, s_a, s_b, k_lds1, k_at0, v_lds0, v_at1);
-      if (j + 1 >= n_tiles) break;
+      if (__builtin_expect(j + 1 >= n_tiles, 0)) break;
       iteration(j + 1, s_b, s_a, k_lds0, k_at1, v_lds1, v_at0);
     }
     wait_loads();  // the fetches past the end of the list must land before the workgroup's LDS is released
