@@ -358,6 +358,65 @@ def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
 # ---------------------------------------------------------------------------
 
 
+def stage_packer_timing(n_blocks=96, n_nodes=2, ranks=8, n_stages=4):
+    """Host side of the planner: one backward-style planning problem (causal block pairs of
+    `n_blocks` query/key blocks over n_nodes x ranks devices) grouped into `n_stages` stages by the
+    native stage packer (dcp_greedy_stage_selection) and, where it has been built from the
+    reference sources into oracle/_ref, by the reference's own C++ module, on the host cores.
+    Reported per greedy-selection call, conversion of the Python containers included for both."""
+    import importlib.util
+
+    from dcp_amd.core import pipeline
+    from oracle import build_ref
+
+    devices = [(n, r) for n in range(n_nodes) for r in range(ranks)]
+    types = ["Q"] * n_blocks + ["KV"] * n_blocks
+    sizes = [1.0 + (i % 7) * 0.25 for i in range(n_blocks)] + [2.0 + (i % 5) * 0.5 for i in range(n_blocks)]
+    for q in range(n_blocks):
+        types += ["OUT", "LSE", "dOUT"]
+        sizes += [sizes[q], sizes[q] / 64, sizes[q]]
+    win, costs = [], []
+    for q in range(n_blocks):
+        for k in range(q + 1):
+            win.append([q, n_blocks + k, 2 * n_blocks + 3 * q, 2 * n_blocks + 3 * q + 1, 2 * n_blocks + 3 * q + 2])
+            costs.append(1.0 + ((q * 31 + k * 17) % 97) / 97.0)
+    home = {i: devices[(i % n_blocks) % len(devices)] for i in range(2 * n_blocks)}
+    for q in range(n_blocks):
+        for j in range(3):
+            home[2 * n_blocks + 3 * q + j] = home[q]
+    w_home = {w: devices[(w * 7) % len(devices)] for w in range(len(win))}
+    dev_work = {d: [] for d in devices}
+    for w, d in w_home.items():
+        dev_work[d].append(w)
+    local0 = {d: {} for d in devices}
+    for i, d in home.items():
+        local0[d][i] = -1
+    total = sum(sizes)
+    target = {d: total / len(devices) / n_stages * 1.2 for d in devices}
+
+    def run(select):
+        scheduled, local = set(), local0
+        t0 = time.perf_counter()
+        for stage in range(n_stages):
+            tgt = target if stage < n_stages - 1 else {d: float("inf") for d in devices}
+            unlocked, _, local = select(set(devices), scheduled, costs, sizes, win, types, dev_work, local, tgt, True,
+                                        stage, None)
+            for ws in unlocked.values():
+                scheduled |= ws
+        assert len(scheduled) == len(win)
+        return (time.perf_counter() - t0) / n_stages * 1e3
+
+    res = {"problem": f"{len(win)} workloads, {len(sizes)} blocks, {len(devices)} devices, {n_stages} stages",
+           "native_ms_per_call": round(min(run(pipeline.greedy_selection_per_device) for _ in range(3)), 3)}
+    ref_path = build_ref.module_path()
+    if ref_path.exists():
+        spec = importlib.util.spec_from_file_location("dcp_cpp", ref_path)
+        ref = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(ref)
+        res["reference_cpp_ms_per_call"] = round(min(run(ref.greedy_selection_per_device) for _ in range(3)), 3)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -424,6 +483,8 @@ def main():
         del ex_f, ex_b
         torch.cuda.empty_cache()
         extra["block_movement"] = movement_microbench()
+    if not args.no_cpu:
+        extra["stage_packer"] = stage_packer_timing()
 
     line = {
         "metric": "mask-aware attn fwd+bwd TFLOP/s @1 MI355X; block merge/gather HBM GB/s",

@@ -35,6 +35,7 @@ SIGNATURES = {
     "dcp_attn_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _F, _I, _P],
     "dcp_attn_bwd": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
     "dcp_attn_bwd_workspace_bytes": [_I, _I, _I, _I, _I],
+    "dcp_greedy_stage_selection": [_I, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P],
 }
 
 _lock = threading.Lock()

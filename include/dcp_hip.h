@@ -257,6 +257,57 @@ int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
 size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
                                     int n_heads_q, int head_dim);
 
+/*
+ * Stage packer of the planner (host code, no GPU work, `stream`-less): decides
+ * which attention blocks ("workloads") every device may run in pipeline stage
+ * `stage_id` and which data blocks must be sent to it first, under a cap on the
+ * bytes each device sends to other nodes in the stage.
+ * Replaces dcp_cpp.greedy_selection_per_device
+ * (csrc/pipeline_generator/pipeline_generator.cpp:19-323, bound in
+ * csrc/interface.cpp:9-11, called from dcp/core/pipeline.py:651-666,703-716).
+ * The reference's sets and dicts of (node, rank) tuples become dense tables;
+ * all pointers are HOST memory:
+ *   device_node[d]               node of device d (devices are 0..n_devices-1)
+ *   workload_costs[w], workload_scheduled[w] (nonzero: already placed in an
+ *                                earlier stage, i.e. the reference's
+ *                                `scheduled_workloads` set)
+ *   input_sizes[i], input_kind[i]  size and DCP_BLOCK_* kind of data block i
+ *                                (the reference's input_block_type_map strings
+ *                                "OUT" / "LSE" / "dOUT", anything else OTHER)
+ *   workload_input_offsets/workload_inputs   CSR of workload_input_map
+ *   device_workload_offsets/device_workloads CSR of device_workload_map
+ *   held_since[d * n_inputs + i] in/out: the stage since which device d holds
+ *                                block i (-1 = from the start), DCP_NOT_HELD if
+ *                                it does not (device_local_inputs_map; updated
+ *                                in place = the third element of the result)
+ *   target_cross_node_load[d]    target_comm_load_per_node
+ * Results: unlocked_by[w] = device that may now run workload w, or -1 (first
+ * element of the reference's result); the transfers (comm_dst[k], comm_input[k],
+ * comm_src[k]) for k < *n_comm in the order they were decided (second element;
+ * n_devices * n_inputs entries always suffice -- on a nonzero return because
+ * `comm_capacity` was too small, *n_comm holds the needed count and held_since
+ * has been modified: call again from the original table); optionally each
+ * device's outgoing cross-node and same-node bytes (what the reference logs).
+ * Where the reference's choice depends on the iteration order of a hash table
+ * (equal compute times, equal sender loads, equal costs) the lowest device
+ * index / workload id wins.
+ */
+#define DCP_BLOCK_OTHER 0
+#define DCP_BLOCK_OUT 1
+#define DCP_BLOCK_LSE 2
+#define DCP_BLOCK_DOUT 3
+#define DCP_NOT_HELD INT32_MIN
+int dcp_greedy_stage_selection(
+    int n_devices, const int32_t* device_node, int n_workloads,
+    const float* workload_costs, const uint8_t* workload_scheduled,
+    int n_inputs, const float* input_sizes, const uint8_t* input_kind,
+    const int32_t* workload_input_offsets, const int32_t* workload_inputs,
+    const int32_t* device_workload_offsets, const int32_t* device_workloads,
+    int32_t* held_since, const float* target_cross_node_load, int is_bw,
+    int stage_id, int32_t* unlocked_by, int32_t* comm_dst, int32_t* comm_input,
+    int32_t* comm_src, int64_t comm_capacity, int64_t* n_comm,
+    float* cross_node_load_out, float* intra_node_load_out);
+
 #ifdef __cplusplus
 }
 #endif
