@@ -33,6 +33,8 @@
 // the per-element range test.
 #include <math.h>
 
+#include <algorithm>
+
 #include "attn_common.h"
 
 namespace dcp {
@@ -64,6 +66,7 @@ struct AttnFwdParams {
   int xcd_group;     // work items per shared K/V stream
   int64_t n_items;   // batch * n_heads_q * q_tiles_per_row
   float scale_log2;  // softmax_scale * log2(e)
+  int* tickets;      // kNumXcd item counters and a count of finished workgroups; zero between launches
 };
 
 // Wave priority by phase: the two waves of a SIMD come from different workgroups and drift
@@ -84,7 +87,7 @@ constexpr float kLazyMax = 8.0f;
 // serves twice the arithmetic; the wave then needs the whole register file (one workgroup
 // per CU, accumulators in the AGPR half).
 template <int DTYPE, int D, int QB>
-__global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
+__device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) {
   constexpr int BN = kFwdBN;
   constexpr int BM = 128 * QB;
   constexpr int KS = D / 16;  // k-steps of S^T = K Q^T
@@ -108,8 +111,7 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
 
   // ---- which (row, head, q tile) ----------------------------------------
   // the query tiles and grouped heads of a row share its K/V: keep them on one XCD
-  int wg = xcd_logical_id(blockIdx.x, p.xcd_group, p.n_items);
-  if (wg < 0) return;
+  int wg = item;
   const int qt = wg % p.q_tiles_per_row;
   wg /= p.q_tiles_per_row;
   const int head = wg % p.n_heads_q;
@@ -555,9 +557,47 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
   }
 }
 
+// The kernel is persistent: the launch has (at most) as many workgroups as the device holds at
+// once and each keeps taking the next work item of its XCD until none is left.  A grid of one
+// workgroup per item loses a tenth of the device to dispatch: workgroup ids are dealt to the 8
+// XCDs strictly in turn, so an XCD with a free slot waits until every XCD before it in the turn
+// has taken its workgroup (13 us between two workgroups of a CU slot on average, against 100 us
+// of work), and the last, unevenly long items leave slots empty at the end.
+//
+// Workgroup b sits on XCD b % 8.  The items that stream the same K/V (the query tiles and grouped
+// heads of a row, `xcd_group` of them with consecutive ids) stay on one XCD: stream s belongs to
+// XCD s % 8, and an XCD's items are handed out in id order (rows come longest first) through one
+// ticket counter per XCD in `p.tickets`.  The counters are zero when the kernel starts; the last
+// workgroup to finish (a ninth counter tells) zeroes them again for the next launch.
+template <int DTYPE, int D, int QB>
+__global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
+  __shared__ int ticket_lds;
+  const int x = blockIdx.x % kNumXcd;
+  const int64_t n_streams = (p.n_items + p.xcd_group - 1) / p.xcd_group;
+  const int64_t n_x = n_streams > x ? (n_streams - x + kNumXcd - 1) / kNumXcd * p.xcd_group : 0;  // items of this XCD
+  while (true) {
+    if (threadIdx.x == 0) ticket_lds = atomicAdd(&p.tickets[x], 1);
+    __syncthreads();
+    const int i = __builtin_amdgcn_readfirstlane(ticket_lds);
+    if (i >= n_x) break;
+    const int64_t item = (x + kNumXcd * (int64_t)(i / p.xcd_group)) * p.xcd_group + i % p.xcd_group;
+    if (item < p.n_items) attn_fwd_item<DTYPE, D, QB>(p, (int)item);
+    __syncthreads();  // the next item reuses the LDS tables and tiles, and the ticket's place
+  }
+  if (threadIdx.x == 0) {
+    const int done = atomicAdd(&p.tickets[kNumXcd], 1);
+    if (done == (int)gridDim.x - 1) {
+#pragma unroll 1
+      for (int j = 0; j <= kNumXcd; ++j) atomicExch(&p.tickets[j], 0);
+    }
+  }
+}
+
 }  // namespace dcp
 
 using namespace dcp;
+
+extern "C" size_t dcp_attn_fwd_workspace_bytes(void) { return 16 * sizeof(int32_t); }
 
 extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                             const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_kv,
@@ -566,7 +606,8 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
                             const int32_t* row_order, int batch, int max_kv_blocks, int total_q,
                             int block_size, int n_heads_q, int n_heads_kv, int head_dim,
                             int64_t kv_slot_stride, int64_t kv_token_stride, int n_out_slots,
-                            float softmax_scale, int dtype, void* stream) {
+                            float softmax_scale, int dtype, void* workspace, size_t workspace_bytes,
+                            void* stream) {
   if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
     return fail(DCP_ERR_UNSUPPORTED, "attn_fwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
   if (head_dim != 64 && head_dim != 128)
@@ -588,6 +629,10 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   DCP_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
                 reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) & 15) == 0,
               "attn_fwd: q/k/v/out must be 16-byte aligned");
+  DCP_REQUIRE(workspace && (reinterpret_cast<uintptr_t>(workspace) & 3) == 0 &&
+                  workspace_bytes >= dcp_attn_fwd_workspace_bytes(),
+              "attn_fwd: workspace of %zu bytes is missing or smaller than the %zu needed", workspace_bytes,
+              dcp_attn_fwd_workspace_bytes());
   AttnFwdParams p;
   p.q = q;
   p.k = k;
@@ -618,8 +663,10 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   p.scale_log2 = softmax_scale * kLog2e;
   p.n_items = (int64_t)batch * n_heads_q * p.q_tiles_per_row;
   p.xcd_group = p.q_tiles_per_row * (n_heads_q / n_heads_kv);
-  const int64_t n_wg = xcd_grid_size(p.n_items, p.xcd_group);
-  DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_fwd: grid too large");
+  DCP_REQUIRE(p.n_items < ((int64_t)1 << 31), "attn_fwd: too many work items");
+  // as many workgroups as the device holds at once (two per CU), a multiple of the XCD count
+  const int64_t n_wg = std::min<int64_t>(xcd_grid_size(p.n_items, 1), xcd_grid_size(2 * (int64_t)device_cu_count(), 1));
+  p.tickets = reinterpret_cast<int*>(workspace);
   dim3 grid((unsigned)n_wg), block(kFwdThreads);
   KernelTimer timer("attn_fwd_kernel", stream);
 #define DCP_FWD(DT, HD) \

@@ -28,6 +28,19 @@ inline int check_launch(const char* what) {
   return DCP_OK;
 }
 
+// Compute units of the current device (asked once per device; 256 if the query fails).
+inline int device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 #define DCP_REQUIRE(cond, ...) \
   do {                         \
     if (!(cond)) return ::dcp::fail(DCP_ERR_ARG, __VA_ARGS__); \

@@ -22,6 +22,7 @@ from dcp_amd.ops.fused_ops import dtype_code
 
 __all__ = [
     "_flash_attn_varlen_forward",
+    "forward_workspace",
     "_flash_attn_varlen_backward",
     "backward_workspace_bytes",
 ]
@@ -31,6 +32,13 @@ def backward_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim) ->
     """Scratch bytes ``_flash_attn_varlen_backward`` needs for these sizes."""
     return int(_lib.load().dcp_attn_bwd_workspace_bytes(
         int(batch), int(total_q), int(block_size), int(n_heads_q), int(head_dim)))
+
+
+def forward_workspace(device="cuda") -> torch.Tensor:
+    """A zeroed work-counter buffer for ``_flash_attn_varlen_forward``.  Every launch leaves it
+    zeroed, so one buffer serves all launches that follow each other on one stream."""
+    n = int(_lib.load().dcp_attn_fwd_workspace_bytes())
+    return torch.zeros((n + 3) // 4, dtype=torch.int32, device=device)
 
 
 def _stream() -> int:
@@ -106,6 +114,7 @@ def _flash_attn_varlen_forward(
     out_=None,
     lse_=None,
     row_order: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None,
 ):
     """Writes the row outputs into ``out_`` / ``lse_`` in place and returns
     ``(out_, lse_, None, None)`` (the reference returns
@@ -116,6 +125,8 @@ def _flash_attn_varlen_forward(
     -1); ``attn_range`` int32 ``[2, total_q]`` or ``[2, 2, total_q]``;
     ``out_`` like q; ``lse_`` fp32 ``[H, n_out_slots, bs]``.
     ``row_order`` (extension): launch order of the rows, longest first.
+    ``workspace`` (extension): a buffer from ``forward_workspace()``; pass one to keep the call
+    allocation-free (e.g. under graph capture), otherwise it is allocated and zeroed here.
     """
     _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap,
                  alibi_slopes, return_softmax)
@@ -136,6 +147,10 @@ def _flash_attn_varlen_forward(
         raise ValueError(f"lse_ shape {tuple(lse_.shape)} does not match out_")
     if softmax_scale is None:
         softmax_scale = head_dim ** (-0.5)
+    if workspace is None:
+        workspace = forward_workspace(q.device)
+    if workspace.dtype != torch.int32 or not workspace.is_contiguous():
+        raise ValueError("workspace must be a contiguous int32 tensor from forward_workspace()")
     _lib.call(
         "dcp_attn_fwd",
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out_.data_ptr(), lse_.data_ptr(),
@@ -149,7 +164,8 @@ def _flash_attn_varlen_forward(
         batch, kv_block_table.shape[1], int(total_q), block_size,
         n_heads_q, n_heads_kv, head_dim,
         kv_slot_stride, kv_token_stride, out_.shape[0],
-        float(softmax_scale), dtype_code(q.dtype), _stream(),
+        float(softmax_scale), dtype_code(q.dtype),
+        workspace.data_ptr(), workspace.numel() * 4, _stream(),
     )
     return out_, lse_, None, None
 

@@ -48,6 +48,7 @@ from dcp_amd.flash_attn_interface import (
     _flash_attn_varlen_backward,
     _flash_attn_varlen_forward,
     backward_workspace_bytes,
+    forward_workspace,
 )
 from dcp_amd.ops.fused_ops import (
     flash_attn_update_out_lse,
@@ -355,6 +356,7 @@ def _prepare_attn(exec: AttentionExecutor, instr: AttnInstr):
         _dev(_pad_block_table(instr.out_block_table), torch.int32),
         _mask_tensor(instr.attn_mask),
         _longest_first(instr.seqlens_kv),
+        forward_workspace(),
     )
 
 
@@ -364,7 +366,7 @@ def _kv_views(kv: torch.Tensor):
 
 def _handle_attn(exec: AttentionExecutor, instr: AttnInstr):
     torch.cuda.nvtx.range_push("AttnInstr")
-    (total_q, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, row_order) = exec._args_cache[
+    (total_q, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, row_order, workspace) = exec._args_cache[
         exec.instr_index
     ]
     k, v = _kv_views(exec.buffers[BufferType.BUFFER_KV])
@@ -387,6 +389,7 @@ def _handle_attn(exec: AttentionExecutor, instr: AttnInstr):
         out_=exec.buffers[BufferType.BUFFER_OUT],
         lse_=exec.buffers[BufferType.BUFFER_LSE],
         row_order=row_order,
+        workspace=workspace,
     )
     torch.cuda.nvtx.range_pop()
 

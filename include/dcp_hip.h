@@ -203,7 +203,15 @@ int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_offsets,
  * NULL = as numbered.  It changes no result.
  * Supported: dtype bf16/fp16, head_dim 64 or 128, block_size % 64 == 0,
  * softmax_scale > 0.
+ * `workspace`: device memory of at least dcp_attn_fwd_workspace_bytes() bytes,
+ * 4-byte aligned, holding the kernel's work counters (the launch is persistent:
+ * its workgroups take (row, head, query tile) items from per-XCD counters).  It
+ * must be ZERO before the first launch that uses it; every launch leaves it
+ * zero again, so one workspace serves any number of launches that follow each
+ * other on a stream (or in a captured graph).  Launches that may run at the
+ * same time need a workspace each.
  */
+size_t dcp_attn_fwd_workspace_bytes(void);
 int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
                  float* lse, const int32_t* cu_seqlens_q,
                  const int32_t* cu_seqlens_kv, const int32_t* attn_range,
@@ -214,7 +222,7 @@ int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
                  int n_heads_q, int n_heads_kv, int head_dim,
                  int64_t kv_slot_stride, int64_t kv_token_stride,
                  int n_out_slots, float softmax_scale, int dtype,
-                 void* stream);
+                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Range-masked, paged, variable-length attention backward.

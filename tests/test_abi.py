@@ -53,12 +53,13 @@ def test_argument_errors_are_reported_without_a_launch(lib):
     with pytest.raises(ValueError, match="Unsupported dtype"):
         _lib.call("dcp_blockwise_sum", 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 128, 7, 0)
     with pytest.raises(ValueError, match="head_dim"):
-        _lib.call("dcp_attn_fwd", *([0] * 8), 1, 0, 0, 0, 0, 1, 1, 64, 64, 1, 1, 96, 0, 0, 1, 1.0, 0, 0)
+        _lib.call("dcp_attn_fwd", *([0] * 8), 1, 0, 0, 0, 0, 1, 1, 64, 64, 1, 1, 96, 0, 0, 1, 1.0, 0, 0, 0, 0)
     with pytest.raises(ValueError, match="bf16 and fp16"):
-        _lib.call("dcp_attn_fwd", *([0] * 8), 1, 0, 0, 0, 0, 1, 1, 64, 64, 1, 1, 128, 0, 0, 1, 1.0, 2, 0)
+        _lib.call("dcp_attn_fwd", *([0] * 8), 1, 0, 0, 0, 0, 1, 1, 64, 64, 1, 1, 128, 0, 0, 1, 1.0, 2, 0, 0, 0)
     # empty problems are accepted and launch nothing
     _lib.call("dcp_fused_copy_varlen", 0, 0, 0, 0, 0, 0, 0, 0, 16, 2, 0)
-    _lib.call("dcp_attn_fwd", *([0] * 8), 1, 0, 0, 0, 0, 0, 1, 0, 64, 1, 1, 128, 0, 0, 1, 1.0, 0, 0)
+    _lib.call("dcp_attn_fwd", *([0] * 8), 1, 0, 0, 0, 0, 0, 1, 0, 64, 1, 1, 128, 0, 0, 1, 1.0, 0, 0, 0, 0)
+    assert lib.dcp_attn_fwd_workspace_bytes() >= 9 * 4
     assert lib.dcp_attn_bwd_workspace_bytes(2, 128, 64, 4, 128) >= 128 * 4 * 4 + 2 * 8 * 4
 
 
