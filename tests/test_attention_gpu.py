@@ -46,6 +46,19 @@ FWD_CASES = {
                              mask_kwargs=dict(block_size=256, k_local=1)),
     "fp16": dict(seqlens=[400, 90], block_size=128, n_heads=4, n_groups=4, head_dim=128, head_block=2,
                  dtype="fp16"),
+    # the masks of the reference's own end-to-end test (tests/runtime/test_flash_attention.py:40-45):
+    # image tokens look forward inside their image (keys AFTER the query position)
+    "multimodal": dict(seqlens=[100 + 200 + 150 + 200 + 90, 64 + 96 + 40], block_size=128, n_heads=4, n_groups=2,
+                       head_dim=128, head_block=2, mask="modality_specific", qkv_scale=0.5,
+                       mask_info=[dict(image_size=200, text_lengths=[100, 150, 90]),
+                                  dict(image_size=96, text_lengths=[64, 40])]),
+    "multimodal_image_to_self": dict(seqlens=[100 + 200 + 150 + 200 + 90], block_size=128, n_heads=4, n_groups=4,
+                                     head_dim=64, head_block=4, mask="modality_specific", qkv_scale=0.5,
+                                     mask_info=[dict(image_size=200, text_lengths=[100, 150, 90])],
+                                     mask_kwargs=dict(limit_image_attn_to_self=True)),
+    "shared_question": dict(seqlens=[1000, 517], block_size=128, n_heads=4, n_groups=2, head_dim=128, head_block=2,
+                            mask="shared_question", qkv_scale=0.5,
+                            mask_kwargs=dict(question_proportion=0.3, n_answers=3)),
 }
 
 
@@ -91,6 +104,9 @@ BWD_CASES = {
                               n_kv_groups=2, kv_split="contiguous"),
     "fp16": dict(seqlens=[400, 90], block_size=128, n_heads=4, n_groups=4, head_dim=128, head_block=2,
                  dtype="fp16", qkv_scale=0.5),
+    "multimodal": FWD_CASES["multimodal"],
+    "multimodal_image_to_self": FWD_CASES["multimodal_image_to_self"],
+    "shared_question": FWD_CASES["shared_question"],
 }
 
 
