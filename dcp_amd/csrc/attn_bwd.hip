@@ -199,17 +199,20 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // the key tiles of a row share its Q/dO tiles: keep them on one XCD
   int wg = xcd_logical_id(blockIdx.x, p.dkv_xcd_group, p.n_dkv_items);
   if (wg < 0) return;
-  const int kt = wg % p.kv_tiles_per_row;
+  // Integer division runs on the vector unit, so its (uniform) results sit in vector registers
+  // and drag every address derived from them there too: each tile load then costs three vector
+  // instructions to rebuild a scalar base.  readfirstlane puts the indices back on the scalar unit.
+  const int kt = __builtin_amdgcn_readfirstlane(wg % p.kv_tiles_per_row);
   wg /= p.kv_tiles_per_row;
-  const int kv_head = wg % p.n_heads_kv;
-  const int bi = wg / p.n_heads_kv;
-  const int b = p.row_order ? p.row_order[bi] : bi;
+  const int kv_head = __builtin_amdgcn_readfirstlane(wg % p.n_heads_kv);
+  const int bi = __builtin_amdgcn_readfirstlane(wg / p.n_heads_kv);
+  const int b = __builtin_amdgcn_readfirstlane(p.row_order ? p.row_order[bi] : bi);
   const int q_begin = p.cu_seqlens_q[b];
   const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
   const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
   const int k0 = kt * BN;
   if (k0 >= seqlen_kv) return;
-  const int blk = k0 / p.block_size;
+  const int blk = __builtin_amdgcn_readfirstlane(k0 / p.block_size);
   const int tok0 = k0 - blk * p.block_size;
   const int group = p.n_heads_q / p.n_heads_kv;
   const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
@@ -528,16 +531,17 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
   // the query tiles and grouped heads of a row share its K/V: keep them on one XCD
   int wg = xcd_logical_id(blockIdx.x, p.dq_xcd_group, p.n_dq_items);
   if (wg < 0) return;
-  const int qt = wg % p.dq_tiles_per_row;
+  // (indices back on the scalar unit after the vector-unit divisions, as in the dK/dV kernel)
+  const int qt = __builtin_amdgcn_readfirstlane(wg % p.dq_tiles_per_row);
   wg /= p.dq_tiles_per_row;
-  const int head = wg % p.n_heads_q;
-  const int bi = wg / p.n_heads_q;
-  const int b = p.row_order ? p.row_order[bi] : bi;
+  const int head = __builtin_amdgcn_readfirstlane(wg % p.n_heads_q);
+  const int bi = __builtin_amdgcn_readfirstlane(wg / p.n_heads_q);
+  const int b = __builtin_amdgcn_readfirstlane(p.row_order ? p.row_order[bi] : bi);
   const int q_begin = p.cu_seqlens_q[b];
   const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
   const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
   if (qt * kDqBM >= seqlen_q) return;
-  const int kv_head = head / (p.n_heads_q / p.n_heads_kv);
+  const int kv_head = __builtin_amdgcn_readfirstlane(head / (p.n_heads_q / p.n_heads_kv));
   const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
   const int q_local = qt * kDqBM + w * 32 + c;
   const bool q_valid = q_local < seqlen_q;

@@ -111,17 +111,20 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 
   // ---- which (row, head, q tile) ----------------------------------------
   // the query tiles and grouped heads of a row share its K/V: keep them on one XCD
+  // Integer division runs on the vector unit, so its (uniform) results sit in vector registers
+  // and drag every address derived from them there too: each tile load then costs three vector
+  // instructions to rebuild a scalar base.  readfirstlane puts the indices back on the scalar unit.
   int wg = item;
-  const int qt = wg % p.q_tiles_per_row;
+  const int qt = __builtin_amdgcn_readfirstlane(wg % p.q_tiles_per_row);
   wg /= p.q_tiles_per_row;
-  const int head = wg % p.n_heads_q;
-  const int bi = wg / p.n_heads_q;
-  const int b = p.row_order ? p.row_order[bi] : bi;
+  const int head = __builtin_amdgcn_readfirstlane(wg % p.n_heads_q);
+  const int bi = __builtin_amdgcn_readfirstlane(wg / p.n_heads_q);
+  const int b = __builtin_amdgcn_readfirstlane(p.row_order ? p.row_order[bi] : bi);
   const int q_begin = p.cu_seqlens_q[b];
   const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
   const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
   if (qt * BM >= seqlen_q) return;
-  const int kv_head = head / (p.n_heads_q / p.n_heads_kv);
+  const int kv_head = __builtin_amdgcn_readfirstlane(head / (p.n_heads_q / p.n_heads_kv));
   const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
 
   int q_local[QB];
