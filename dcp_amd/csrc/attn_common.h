@@ -273,6 +273,21 @@ inline int64_t xcd_grid_size(int64_t total, int group) {
   return (total + per_super - 1) / per_super * per_super;
 }
 
+// A persistent kernel's item body reads the kernel arguments through a pointer to the
+// kernel-argument segment that is made opaque once per item, so that the compiler loads each
+// field where the item uses it.  Read through the kernel's by-value parameter, every field an
+// item's prologue needs is loaded once before the item loop and then occupies a scalar register
+// through the whole matrix loop (the kernels end up at the scalar register limit).
+// The kernel must have the parameter struct as its only argument.
+template <typename Params>
+using KernArgs = const __attribute__((address_space(4))) Params;
+template <typename Params>
+__device__ __forceinline__ KernArgs<Params>& fresh_kernel_args() {
+  KernArgs<Params>* args = (KernArgs<Params>*)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(args));
+  return *args;
+}
+
 // Workgroup barrier between the phases of a kernel whose LDS tiles are filled
 // by global_load_lds.  It waits for this wave's LDS accesses (lgkmcnt) but, unlike
 // __syncthreads(), not for its outstanding global loads, so tiles requested a phase
