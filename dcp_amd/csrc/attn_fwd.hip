@@ -66,7 +66,7 @@ struct AttnFwdParams {
   int xcd_group;     // work items per shared K/V stream
   int64_t n_items;   // batch * n_heads_q * q_tiles_per_row
   float scale_log2;  // softmax_scale * log2(e)
-  int* tickets;      // kNumXcd item counters and a count of finished workgroups; zero between launches
+  int* tickets;      // kNumXcd item counters, zeroed before the launch
 };
 
 // Wave priority by phase: the two waves of a SIMD come from different workgroups and drift
@@ -570,8 +570,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 // Workgroup b sits on XCD b % 8.  The items that stream the same K/V (the query tiles and grouped
 // heads of a row, `xcd_group` of them with consecutive ids) stay on one XCD: stream s belongs to
 // XCD s % 8, and an XCD's items are handed out in id order (rows come longest first) through one
-// ticket counter per XCD in `p.tickets`.  The counters are zero when the kernel starts; the last
-// workgroup to finish (a ninth counter tells) zeroes them again for the next launch.
+// ticket counter per XCD in `p.tickets`, which a one-wave kernel zeroes on the stream just before.
 template <int DTYPE, int D, int QB>
 __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
   __shared__ int ticket_lds;
@@ -587,13 +586,10 @@ __global__ __launch_bounds__(kFwdThreads, QB == 1 ? 2 : 1) void attn_fwd_kernel(
     if (item < p.n_items) attn_fwd_item<DTYPE, D, QB>(p, (int)item);
     __syncthreads();  // the next item reuses the LDS tables and tiles, and the ticket's place
   }
-  if (threadIdx.x == 0) {
-    const int done = atomicAdd(&p.tickets[kNumXcd], 1);
-    if (done == (int)gridDim.x - 1) {
-#pragma unroll 1
-      for (int j = 0; j <= kNumXcd; ++j) atomicExch(&p.tickets[j], 0);
-    }
-  }
+}
+
+__global__ void attn_fwd_reset_tickets_kernel(int* tickets) {
+  if (threadIdx.x < kNumXcd) tickets[threadIdx.x] = 0;
 }
 
 }  // namespace dcp
@@ -671,6 +667,7 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   const int64_t n_wg = std::min<int64_t>(xcd_grid_size(p.n_items, 1), xcd_grid_size(2 * (int64_t)device_cu_count(), 1));
   p.tickets = reinterpret_cast<int*>(workspace);
   dim3 grid((unsigned)n_wg), block(kFwdThreads);
+  hipLaunchKernelGGL(attn_fwd_reset_tickets_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, p.tickets);
   KernelTimer timer("attn_fwd_kernel", stream);
 #define DCP_FWD(DT, HD) \
   hipLaunchKernelGGL((attn_fwd_kernel<DT, HD, 1>), grid, block, 0, (hipStream_t)stream, p)

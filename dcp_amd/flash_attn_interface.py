@@ -35,10 +35,10 @@ def backward_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim) ->
 
 
 def forward_workspace(device="cuda") -> torch.Tensor:
-    """A zeroed work-counter buffer for ``_flash_attn_varlen_forward``.  Every launch leaves it
-    zeroed, so one buffer serves all launches that follow each other on one stream."""
+    """A work-counter buffer for ``_flash_attn_varlen_forward`` (contents are overwritten by
+    every launch); one buffer serves all launches that follow each other on one stream."""
     n = int(_lib.load().dcp_attn_fwd_workspace_bytes())
-    return torch.zeros((n + 3) // 4, dtype=torch.int32, device=device)
+    return torch.empty((n + 3) // 4, dtype=torch.int32, device=device)
 
 
 def _stream() -> int:
@@ -126,7 +126,7 @@ def _flash_attn_varlen_forward(
     ``out_`` like q; ``lse_`` fp32 ``[H, n_out_slots, bs]``.
     ``row_order`` (extension): launch order of the rows, longest first.
     ``workspace`` (extension): a buffer from ``forward_workspace()``; pass one to keep the call
-    allocation-free (e.g. under graph capture), otherwise it is allocated and zeroed here.
+    allocation-free (e.g. under graph capture), otherwise it is allocated here.
     """
     _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap,
                  alibi_slopes, return_softmax)

@@ -203,13 +203,13 @@ int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_offsets,
  * NULL = as numbered.  It changes no result.
  * Supported: dtype bf16/fp16, head_dim 64 or 128, block_size % 64 == 0,
  * softmax_scale > 0.
- * `workspace`: device memory of at least dcp_attn_fwd_workspace_bytes() bytes,
- * 4-byte aligned, holding the kernel's work counters (the launch is persistent:
- * its workgroups take (row, head, query tile) items from per-XCD counters).  It
- * must be ZERO before the first launch that uses it; every launch leaves it
- * zero again, so one workspace serves any number of launches that follow each
- * other on a stream (or in a captured graph).  Launches that may run at the
- * same time need a workspace each.
+ * `workspace`: caller-provided device scratch of at least
+ * dcp_attn_fwd_workspace_bytes() bytes, 4-byte aligned, for the kernel's work
+ * counters (the launch is persistent: its workgroups take (row, head, query
+ * tile) items from per-XCD counters).  Its contents are overwritten (a small
+ * kernel zeroes it on `stream` before the attention kernel); one workspace
+ * serves any number of launches that follow each other on a stream or in a
+ * captured graph, launches that may run at the same time need one each.
  */
 size_t dcp_attn_fwd_workspace_bytes(void);
 int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,

@@ -122,27 +122,26 @@ def test_backward_matches_dense_truth(gpu, name):
     assert e_dkv <= GRAD_ATOL, e_dkv
 
 
-def test_forward_work_counters_are_left_zero_and_reusable(gpu):
-    """The forward kernel hands out work items through counters in a caller workspace; a launch
-    must leave them zero so that the next launch (here: the same plan, three times, multi-partial
-    so several attention launches share the workspace per run) starts clean."""
-    from dcp_amd.flash_attn_interface import _flash_attn_varlen_forward, forward_workspace
-
+def test_forward_workspace_is_reusable_and_may_hold_anything(gpu):
+    """The forward kernel hands out work items through counters in a caller workspace that each
+    launch resets itself: a workspace full of garbage, reused by every attention launch of a
+    multi-partial plan and over repeated runs, changes nothing."""
     case = make_case(**FWD_CASES["c1_every_block_its_own_partial"])
     res, ex = run_executor(case)
     _check_forward(case, res)
+    spaces = [a[-1] for a in ex._args_cache.values() if isinstance(a, tuple) and isinstance(a[-1], torch.Tensor)
+              and a[-1].dtype == torch.int32 and a[-1].numel() <= 64]
+    assert spaces, "the prepared attention instructions carry their workspaces"
     layout = case["layout"]
     lq = layout.to_local_q(case["q"]).cuda()
     lkv = layout.to_local_kv(case["kv"]).cuda()
-    for _ in range(2):
+    for fill in (0x7fffffff, -5):
+        for w in spaces:
+            w.fill_(fill)
         out, lse = ex.forward(lq, lkv)
         torch.cuda.synchronize()
         again = [layout.from_local_q(out.cpu()), layout.from_local_lse(lse.cpu())]
         assert torch.equal(again[0], res[0]) and torch.equal(again[1], res[1])
-    spaces = [a[-1] for a in ex._args_cache.values() if isinstance(a, tuple) and isinstance(a[-1], torch.Tensor)
-              and a[-1].dtype == torch.int32 and a[-1].numel() == forward_workspace().numel()]
-    assert spaces, "the prepared attention instructions carry their workspaces"
-    assert all(int(w.abs().sum()) == 0 for w in spaces)
     # a missing workspace is an argument error, reported before anything is launched
     from dcp_amd import _lib
 
