@@ -74,5 +74,23 @@ def build(verbose: bool = True) -> Path:
     return LIB_PATH
 
 
+HOST_CHECK_SRC = PKG_DIR.parent / "tests" / "abi_host" / "abi_host_check.cpp"
+HOST_CHECK_BIN = HOST_CHECK_SRC.with_suffix("")
+
+
+def build_abi_host_check(verbose: bool = True) -> Path:
+    """Compiles the plain C++ host program of tests/abi_host against the built library (it
+    includes only include/dcp_hip.h and the HIP runtime).  The GPU test runs the binary."""
+    cmd = [HIPCC, f"--offload-arch={ARCH}", "-O2", "-std=c++17", f"-I{INCLUDE}", str(HOST_CHECK_SRC),
+           "-o", str(HOST_CHECK_BIN), f"-L{LIB_PATH.parent}", "-ldcp_hip", "-Wl,-rpath,$ORIGIN/../../dcp_amd", f"-Wl,-rpath,{LIB_PATH.parent}"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"host check failed to build:\n{proc.stderr}")
+    if verbose:
+        print(f"built {HOST_CHECK_BIN}", file=sys.stderr)
+    return HOST_CHECK_BIN
+
+
 if __name__ == "__main__":
     build()
+    build_abi_host_check()
