@@ -60,6 +60,7 @@ struct AttnBwdParams {
   void* dk;
   void* dv;
   float* delta;      // [total_q, H]
+  float* lse2;       // [total_q, H]: lse * log2(e), written by the prep kernel for the dK/dV kernel
   int32_t* hull;     // [batch * q_tiles_per_row, 8]
   int* tickets;      // work-item counters of the persistent dQ kernel (kTicketInts); zeroed by the hull kernel
   const int32_t* cu_seqlens_q;
@@ -127,7 +128,12 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const AttnBwdParams p) {
 #pragma unroll
   for (int o2 = LPR / 2; o2 > 0; o2 >>= 1) acc += __shfl_xor(acc, o2);
   const int64_t qrow = ((int64_t)(q_begin + t) * p.n_heads_q + hd);
-  if (g == 0) p.delta[qrow] = acc;
+  if (g == 0) {
+    p.delta[qrow] = acc;
+    // the log-sum-exp in the base-2 domain the kernels work in, one multiply per (token, head)
+    // here instead of one per (query, key tile) in the dK/dV kernel's vector phase
+    p.lse2[qrow] = p.lse[((int64_t)hd * p.n_out_slots + p.out_block_table[b]) * p.block_size + t] * kLog2e;
+  }
 }
 
 // One wave per (row, 64-query tile).  hull[0..3] = lo0, hi0, lo1, hi1 over
@@ -309,11 +315,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const bool role_rng = w < 2, role_lse = w == 2;
   const int sc_plane = p.n_ranges == 2 ? 2 * w : 0;
   const char* sc_base0 = role_rng   ? reinterpret_cast<const char*>(p.attn_range + (int64_t)sc_plane * p.total_q + q_begin)
-                         : role_lse ? reinterpret_cast<const char*>(p.lse + (int64_t)o_slot * p.block_size)
+                         : role_lse ? reinterpret_cast<const char*>(p.lse2 + (int64_t)q_begin * p.n_heads_q)
                                     : reinterpret_cast<const char*>(p.delta + (int64_t)q_begin * p.n_heads_q);
-  const int64_t sc_head_bytes = role_rng ? 0 : role_lse ? (int64_t)p.n_out_slots * p.block_size * 4 : 4;
+  const int64_t sc_head_bytes = role_rng ? 0 : 4;
   const int64_t sc_second_bytes = role_rng ? (int64_t)p.total_q * 4 : 0;
-  const int sc_query_bytes = (role_rng || role_lse) ? 4 : p.n_heads_q * 4;
+  const int sc_query_bytes = role_rng ? 4 : p.n_heads_q * 4;
   const uint32_t sc_at0 = role_rng ? rng_at + (2 * w * BM) * 4 : role_lse ? lse_at : delta_at;
   const uint32_t sc_at_stage = role_rng ? 4 * BM * 4 : BM * 4, sc_at_second = role_rng ? BM * 4 : 0;
   auto request_scalars = [&](int head, int qt, int st) {
@@ -433,7 +439,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       float pv[4], dsv[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -kLog2e * l4[r]));  // masked: exp2(-inf) = 0
+        pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));  // l4: lse * log2(e); masked: exp2(-inf) = 0
         dsv[r] = pv[r] * (dp_acc[4 * g + r] - d4[r]);
       }
       pb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(pv[0], pv[1]);
@@ -824,7 +830,7 @@ extern "C" size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block
   if (batch < 0 || total_q < 0 || block_size <= 0 || n_heads_q <= 0 || head_dim <= 0) return 0;
   const size_t q_tiles = (size_t)batch * ((block_size + kBwdBM - 1) / kBwdBM);
   (void)head_dim;
-  return align256((size_t)total_q * n_heads_q * sizeof(float)) + align256(q_tiles * 8 * sizeof(int32_t)) +
+  return 2 * align256((size_t)total_q * n_heads_q * sizeof(float)) + align256(q_tiles * 8 * sizeof(int32_t)) +
          align256(kTicketInts * sizeof(int32_t));
 }
 
@@ -883,6 +889,8 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
   p.dv = dv;
   char* ws = reinterpret_cast<char*>(workspace);
   p.delta = reinterpret_cast<float*>(ws);
+  ws += align256((size_t)total_q * n_heads_q * sizeof(float));
+  p.lse2 = reinterpret_cast<float*>(ws);
   ws += align256((size_t)total_q * n_heads_q * sizeof(float));
   p.hull = reinterpret_cast<int32_t*>(ws);
   ws += align256((size_t)batch * ((block_size + kBwdBM - 1) / kBwdBM) * 8 * sizeof(int32_t));

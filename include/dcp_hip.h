@@ -258,8 +258,9 @@ int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                  void* stream);
 
 /*
- * Bytes of scratch dcp_attn_bwd needs for these sizes: rowsum(dO*O)
- * (total_q*n_heads_q floats) and the per-(row, 64-query tile) range hulls.  No counterpart in the reference (its
+ * Bytes of scratch dcp_attn_bwd needs for these sizes: rowsum(dO*O) and the
+ * base-2 log-sum-exp (total_q*n_heads_q floats each), the per-(row, 64-query
+ * tile) range hulls and the dQ kernel's work counters.  No counterpart in the reference (its
  * flash-attention fork allocates these inside the call).
  */
 size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
