@@ -2,7 +2,7 @@
 //
 // Two small kernels and two big ones per call:
 //
-//   bwd_prep_kernel      delta[q, h] = sum_d dO*O
+//   bwd_prep_kernel      delta[q, h] = -sum_d dO*O  (negated: it is added, as an accumulator's initial value)
 //   bwd_tile_hull_kernel per (row, 64-query tile): hull and core of the rows'
 //                        key ranges, so the dK/dV kernel can skip / unmask tiles
 //   attn_bwd_dkv_kernel  key-outer: one workgroup per (row, 64-key tile, kv
@@ -59,7 +59,7 @@ struct AttnBwdParams {
   void* dq;
   void* dk;
   void* dv;
-  float* delta;      // [total_q, H]
+  float* delta;      // [total_q, H]: MINUS rowsum(dO * O)
   float* lse2;       // [total_q, H]: lse * log2(e), written by the prep kernel for the dK/dV kernel
   int32_t* hull;     // [batch * q_tiles_per_row, 8]
   int* tickets;      // work-item counters of the persistent dQ kernel (kTicketInts); zeroed by the hull kernel
@@ -101,7 +101,7 @@ constexpr int kBwdThreads = 256;
 constexpr int kTicketInts = 16;  // one counter per XCD (the rest unused)
 
 // ---------------------------------------------------------------------------
-// delta[q, h] = sum_d dO*O.  LPR lanes per (token, head) row, 8 elements each.
+// delta[q, h] = -sum_d dO*O.  LPR lanes per (token, head) row, 8 elements each.
 // grid: (batch, row chunks)
 // ---------------------------------------------------------------------------
 template <int DTYPE, int D>
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const AttnBwdParams p) {
   for (int o2 = LPR / 2; o2 > 0; o2 >>= 1) acc += __shfl_xor(acc, o2);
   const int64_t qrow = ((int64_t)(q_begin + t) * p.n_heads_q + hd);
   if (g == 0) {
-    p.delta[qrow] = acc;
+    p.delta[qrow] = -acc;
     // the log-sum-exp in the base-2 domain the kernels work in, one multiply per (token, head)
     // here instead of one per (query, key tile) in the dK/dV kernel's vector phase
     p.lse2[qrow] = p.lse[((int64_t)hd * p.n_out_slots + p.out_block_table[b]) * p.block_size + t] * kLog2e;
@@ -391,8 +391,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         __builtin_amdgcn_sched_barrier(0);  // one group's planes in registers at a time
       }
     }
+    // dP starts from -delta of its query (dS = P (dP - delta)): the subtraction rides on the
+    // accumulation instead of costing a vector instruction per element afterwards
 #pragma unroll
-    for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][qi * 32 + 8 * g + 4 * h]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) dp_acc[4 * g + r] = d4[r];
+    }
     // Everything the step's 32 MFMAs read from LDS forms one stream, read AHEAD entries ahead
     // into four rotating registers, across both matrix phases (the first operands of the second
     // phase are on their way while the vector phase runs):
@@ -435,12 +441,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     for (int g = 0; g < 4; ++g) {
       const int qrow = qi * 32 + 8 * g + 4 * h;
       const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[st][qrow]);
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][qrow]);
       float pv[4], dsv[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));  // l4: lse * log2(e); masked: exp2(-inf) = 0
-        dsv[r] = pv[r] * (dp_acc[4 * g + r] - d4[r]);
+        dsv[r] = pv[r] * dp_acc[4 * g + r];
       }
       pb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(pv[0], pv[1]);
       pb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(pv[2], pv[3]);
@@ -628,6 +633,12 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) dq_acc[dt][i] = 0.0f;
+  // dP^T starts from -delta of the lane's query (dS = P (dP - delta)): a register block that
+  // holds it serves as the C operand of the first MFMA of every dP^T chain, so the subtraction
+  // costs no vector instruction per element
+  f32x16 dp_init;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) dp_init[i] = delta;
 
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint16_t* vg = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)kv_head * D;
@@ -677,8 +688,6 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
 #pragma unroll
         for (int i = 0; i < 16; ++i) s_acc[i] = rng.contains(kb + 8 * (i / 4) + (i % 4)) ? 0.0f : -INFINITY;
       }
-#pragma unroll
-      for (int i = 0; i < 16; ++i) dp_acc[i] = 0.0f;
       // operands four k-steps at a time; the two accumulation chains interleave
 #pragma unroll
       for (int half = 0; half < KS / 4; ++half) {
@@ -690,7 +699,7 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
 #pragma unroll
         for (int k4 = 0; k4 < 4; ++k4) {
           s_acc = mfma_32x32x16<DTYPE>(ka[k4], qreg[half * 4 + k4], s_acc);
-          dp_acc = mfma_32x32x16<DTYPE>(va[k4], doreg[half * 4 + k4], dp_acc);
+          dp_acc = mfma_32x32x16<DTYPE>(va[k4], doreg[half * 4 + k4], half == 0 && k4 == 0 ? dp_init : dp_acc);
         }
         // one tile load per group of eight MFMAs: 2 * KS / 4 of the NL here, the rest below
         if (nt * (KS / 4) + half < NL / 2) issue_load(nt * (KS / 4) + half);
@@ -702,7 +711,7 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
         for (int j = 0; j < 8; ++j) {
           const int i = g * 8 + j;
           const float pr = fast_exp2(fmaf(s_acc[i], p.scale_log2, -lse2));  // masked: exp2(-inf) = 0
-          e[j] = pr * (dp_acc[i] - delta);
+          e[j] = pr * dp_acc[i];
         }
         u32x4 packed = {pack2<DTYPE>(e[0], e[1]), pack2<DTYPE>(e[2], e[3]), pack2<DTYPE>(e[4], e[5]),
                         pack2<DTYPE>(e[6], e[7])};
