@@ -65,16 +65,28 @@ __device__ __forceinline__ float halves_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-__device__ __forceinline__ int wave_min(int x) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) x = min(x, __shfl_xor(x, o));
-  return __builtin_amdgcn_readfirstlane(x);  // the same in every lane: let the compiler know
+// Minimum / maximum over the wave, as a scalar.  Four DPP steps (row_shr 1, 2, 4, 8) leave each
+// 16-lane row's result in its last lane; the four row results are combined on the scalar unit.
+// (Butterfly shuffles would be six dependent trips through LDS each, and a workgroup's prologue
+// takes eight of these reductions.)
+template <bool IS_MIN>
+__device__ __forceinline__ int wave_reduce_minmax(int x) {
+#define DCP_DPP_STEP(ctrl)                                                       \
+  {                                                                              \
+    const int y = __builtin_amdgcn_update_dpp(x, x, ctrl, 0xf, 0xf, false);      \
+    x = IS_MIN ? min(x, y) : max(x, y);                                          \
+  }
+  DCP_DPP_STEP(0x111)  // row_shr:1 (a lane without a source keeps its own value)
+  DCP_DPP_STEP(0x112)  // row_shr:2
+  DCP_DPP_STEP(0x114)  // row_shr:4
+  DCP_DPP_STEP(0x118)  // row_shr:8
+#undef DCP_DPP_STEP
+  const int r0 = __builtin_amdgcn_readlane(x, 15), r1 = __builtin_amdgcn_readlane(x, 31);
+  const int r2 = __builtin_amdgcn_readlane(x, 47), r3 = __builtin_amdgcn_readlane(x, 63);
+  return IS_MIN ? min(min(r0, r1), min(r2, r3)) : max(max(r0, r1), max(r2, r3));
 }
-__device__ __forceinline__ int wave_max(int x) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) x = max(x, __shfl_xor(x, o));
-  return __builtin_amdgcn_readfirstlane(x);
-}
+__device__ __forceinline__ int wave_min(int x) { return wave_reduce_minmax<true>(x); }
+__device__ __forceinline__ int wave_max(int x) { return wave_reduce_minmax<false>(x); }
 
 // Row index (within a 32-row MFMA tile) of accumulator element i for a lane
 // in half h.
