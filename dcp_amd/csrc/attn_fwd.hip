@@ -81,6 +81,11 @@ constexpr int kFwdThreads = 256;
 // accumulators that costs no accuracy, and it takes the rescale (64 multiplies per query
 // block) out of almost every tile after a row's first few.
 constexpr float kLazyMax = 8.0f;
+// On the fast path a tile is exponentiated against the row's current reference without taking
+// its maximum first; it is redone against a raised reference only if one lane's partial row sum
+// of the tile (32 weights) reaches kMaxTileSum, i.e. if some weight might exceed it.  2^14 keeps
+// every accepted weight representable in fp16 and far from overflowing the fp32 accumulators.
+constexpr float kMaxTileSum = 16384.0f;
 
 // QB = 32-row query blocks per wave: the workgroup owns 128*QB query rows.  With QB = 2 every
 // K / V^T operand read from LDS feeds two matrix instructions and every tile brought into LDS
@@ -314,39 +319,25 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
   float alpha[QB];       // pending rescale of O^T (applied before the tile's P^T is multiplied in)
   bool rescale[QB];
   float m_use[QB], lsum[QB];
-  // The row maximum of a tile is taken in kMaxParts pieces of 32 / kMaxParts elements and
-  // a final step, so that it can be spread between matrix instructions.
-  constexpr int kMaxParts = 4;
-  float mx_part[QB];
-  auto row_max_part = [&](const f32x16 (&sc)[2][QB], int qb, int part) {
-    constexpr int PER = 32 / kMaxParts;
-    float mx = part == 0 ? -INFINITY : mx_part[qb];
-#pragma unroll
-    for (int i = 0; i < PER; ++i) mx = fmaxf(mx, sc[(part * PER + i) >> 4][qb][(part * PER + i) & 15]);
-    mx_part[qb] = mx;
-  };
-  // `valid` false (the accumulators hold no tile): as if every element were masked, nothing changes
-  auto row_max_finish = [&](int qb, bool valid) {
-    float mx = valid ? mx_part[qb] * p.scale_log2 : -INFINITY;  // -inf stays -inf (scale > 0)
-    mx = halves_max(mx);
-    // raise the reference maximum only when the tile exceeds it by more than kLazyMax (always
-    // for a row that had none yet: -inf + kLazyMax = -inf), then for every row of the wave
-    rescale[qb] = __any(mx > m_run[qb] + kLazyMax);
-    const float m_new = rescale[qb] ? fmaxf(m_run[qb], mx) : m_run[qb];
-    m_use[qb] = (m_new == -INFINITY) ? 0.0f : m_new;
-    alpha[qb] = fast_exp2(m_run[qb] - m_use[qb]);  // m_run = -inf -> 0; 1 where the maximum stays
-    l_run[qb] *= alpha[qb];
-    m_run[qb] = m_new;
-    lsum[qb] = 0.0f;
-  };
-  // The maximum step of tile j+1 runs at the end of iteration j (inside O^T += V^T P^T of tile j
-  // on the fast path), off the head of the exponentials' dependency chain.
+  // The maximum step of a tile: the row maximum, and the row's reference raised to it if needed.
   auto softmax_max = [&](const f32x16 (&sc)[2][QB]) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
+      float mx = -INFINITY;
 #pragma unroll
-      for (int part = 0; part < kMaxParts; ++part) row_max_part(sc, qb, part);
-      row_max_finish(qb, true);
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[nt][qb][e]);
+      mx = halves_max(mx * p.scale_log2);  // -inf stays -inf (scale > 0)
+      // raise the reference maximum only when the tile exceeds it by more than kLazyMax (always
+      // for a row that had none yet: -inf + kLazyMax = -inf), then for every row of the wave
+      rescale[qb] = __any(mx > m_run[qb] + kLazyMax);
+      const float m_new = rescale[qb] ? fmaxf(m_run[qb], mx) : m_run[qb];
+      m_use[qb] = (m_new == -INFINITY) ? 0.0f : m_new;
+      alpha[qb] = fast_exp2(m_run[qb] - m_use[qb]);  // m_run = -inf -> 0; 1 where the maximum stays
+      l_run[qb] *= alpha[qb];
+      m_run[qb] = m_new;
+      lsum[qb] = 0.0f;
     }
   };
   // elements 2*c2, 2*c2+1 of the 32 this lane holds for query block qb
@@ -411,14 +402,11 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
       if ((i + 1) % (N / KTile::LPW) == 0) issue_load(i / (N / KTile::LPW));
       __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) l_run[qb] += lsum[qb];
   };
 
   // O^T += V^T P^T: V^T comes out of the row-major V tile by transpose loads, read
-  // two operands ahead; consecutive MFMAs go to different accumulators.  The row maxima of the
-  // next tile (S^T in s_next if has_next) are taken between the first MFMAs.
-  auto multiply_pv = [&](const uint16_t* v_lds, const f32x16 (&s_next)[2][QB], bool has_next) {
+  // two operands ahead; consecutive MFMAs go to different accumulators
+  auto multiply_pv = [&](const uint16_t* v_lds) {
     constexpr int N = 4 * DT;
     constexpr int AHEAD = 2;
     auto v_operand = [&](int i) { return VTile::template read_col<true>(v_lds, v_rd, i / DT, i % DT); };
@@ -431,17 +419,6 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
         o_acc[qb][i % DT] = mfma_32x32x16<DTYPE>(va[i & 3], pb[qb][i / DT], o_acc[qb][i % DT]);
-      {
-        // a piece after every second MFMA
-        constexpr int STEP = N >= 2 * (kMaxParts + 1) ? 2 : 1;
-        if (i % STEP == STEP - 1 && i / STEP <= kMaxParts) {
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) {
-            if (i / STEP < kMaxParts) row_max_part(s_next, qb, i / STEP);
-            else row_max_finish(qb, has_next);
-          }
-        }
-      }
       if ((i + 1) % (N / VTile::LPW) == 0) issue_load(KTile::LPW + i / (N / VTile::LPW));
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -461,6 +438,8 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
   int tile_cur = 0, tile_nxt = 0;  // key tile numbers of list entries j and j+1
   int64_t v_off = 0;               // offset of list entry j+1 (its V is requested in iteration j)
   bool cur_full = false;           // list entry j lies inside every row's range
+  bool pending = false;            // the maximum step of list entry j has been done already
+  bool anchored = false;           // every row of the wave has a (finite) reference maximum
   auto iteration = [&](int j, f32x16 (&s_cur)[2][QB], f32x16 (&s_nxt)[2][QB], const uint16_t* k_nxt, uint32_t k_fill,
                        const uint16_t* v_cur, uint32_t v_fill) {
     __builtin_amdgcn_s_waitcnt(0);
@@ -472,32 +451,57 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
     // the S^T product carries the K loads, O^T += V^T P^T the V loads; a wave that skips one
     // of them still has its share of the tile to request
     const bool nxt_full = j + 1 < n_tiles && tile_is_full(tile_nxt);
-    bool cur = true, nxt = true;
-    if (__builtin_expect(cur_full && nxt_full, 1)) {
-      // the common case, decided by one test per iteration: this tile and the next are
-      // inside every row's range
+    bool cur = true;
+    if (__builtin_expect(cur_full && nxt_full && anchored, 1)) {
+      // The common case, decided by one test per iteration: this tile and the next are inside
+      // every row's range and every row has a reference maximum.  The weights are taken relative
+      // to that reference WITHOUT looking at the tile's own maximum first ...
+      if (!pending) {
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          lsum[qb] = 0.0f;
+          rescale[qb] = false;
+        }
+      }
       __builtin_amdgcn_s_setprio(kPrioFused);
       multiply_qk_with_softmax(k_nxt, s_nxt, s_cur);
+      // ... and the tile's partial row sums tell afterwards whether that was safe: every weight is
+      // at most its lane's sum.  Only if a sum is out of bounds (or not a number) is the tile's
+      // maximum taken, the reference raised and the tile exponentiated again.
+      bool redo = false;
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) redo |= __any(!(lsum[qb] < kMaxTileSum));
+      if (__builtin_expect(redo, 0)) {
+        softmax_max(s_cur);
+        softmax(s_cur);
+      } else {
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) l_run[qb] += lsum[qb];
+      }
     } else {
       cur = cur_full || wave_sees(tile_cur);
-      nxt = j + 1 < n_tiles && (nxt_full || wave_sees(tile_nxt));
+      const bool nxt = j + 1 < n_tiles && (nxt_full || wave_sees(tile_nxt));
       if (nxt) {
         multiply_qk(tile_nxt, k_nxt, s_nxt);
       } else {
 #pragma unroll
         for (int i = 0; i < KTile::LPW; ++i) issue_load(i);
       }
-      if (cur) softmax(s_cur);
+      if (cur) {
+        if (!pending) softmax_max(s_cur);
+        softmax(s_cur);
+        anchored |= cur_full;  // a tile every row sees gives every row a reference
+      }
     }
+    pending = false;
     if (__builtin_expect(cur, 1)) {
       apply_rescale();
       __builtin_amdgcn_s_setprio(kPrioDense);
-      multiply_pv(v_cur, s_nxt, nxt);
+      multiply_pv(v_cur);
       __builtin_amdgcn_s_setprio(kPrioControl);
     } else {
 #pragma unroll
       for (int i = 0; i < VTile::LPW; ++i) issue_load(KTile::LPW + i);
-      if (nxt) softmax_max(s_nxt);
     }
     cur_full = nxt_full;
     tile_cur = tile_nxt;
@@ -527,6 +531,8 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
     if (wave_sees(tile_cur)) {
       multiply_qk(tile_cur, k_lds0, s_a);
       softmax_max(s_a);
+      pending = true;
+      anchored = cur_full;
     }
     for (int j = 0; j < n_tiles; j += 2) {
       iteration(j, s_a, s_b, k_lds1, k_at0, v_lds0, v_at1);

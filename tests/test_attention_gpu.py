@@ -20,8 +20,11 @@ def _check_forward(case, res):
     out, lse = res[0].float().numpy(), res[1].numpy()
     t_out, t_lse = dense_truth(case)
     assert np.isfinite(lse).all()
-    assert np.abs(out - t_out).max() <= OUT_TOL, np.abs(out - t_out).max()
-    assert np.abs(lse - t_lse).max() <= LSE_TOL, np.abs(lse - t_lse).max()
+    # absolute for |out| <= 1, relative above (one bf16 ulp exceeds the absolute bound from |out| = 4 on)
+    e_out = (np.abs(out - t_out) / np.maximum(1.0, np.abs(t_out))).max()
+    assert e_out <= OUT_TOL, e_out
+    e_lse = (np.abs(lse - t_lse) / np.maximum(1.0, np.abs(t_lse) / 16.0)).max()  # fp32 lse: ~1e-7 relative
+    assert e_lse <= LSE_TOL, e_lse
 
 
 FWD_CASES = {
@@ -59,6 +62,12 @@ FWD_CASES = {
     "shared_question": dict(seqlens=[1000, 517], block_size=128, n_heads=4, n_groups=2, head_dim=128, head_block=2,
                             mask="shared_question", qkv_scale=0.5,
                             mask_kwargs=dict(question_proportion=0.3, n_answers=3)),
+    # scores spread over +-60 in the base-2 domain: later tiles keep exceeding the running reference
+    # maximum by far more than the kernel's fast path tolerates, so its redo branch is exercised
+    "large_scores": dict(seqlens=[2048, 700], block_size=256, n_heads=4, n_groups=2, head_dim=128, head_block=2,
+                         qkv_scale=3.0),
+    "large_scores_fp16": dict(seqlens=[1536], block_size=256, n_heads=2, n_groups=2, head_dim=64, head_block=2,
+                              qkv_scale=3.0, dtype="fp16"),
 }
 
 
