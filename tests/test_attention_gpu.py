@@ -62,6 +62,9 @@ FWD_CASES = {
     "shared_question": dict(seqlens=[1000, 517], block_size=128, n_heads=4, n_groups=2, head_dim=128, head_block=2,
                             mask="shared_question", qkv_scale=0.5,
                             mask_kwargs=dict(question_proportion=0.3, n_answers=3)),
+    # the smallest block the kernels take (one query tile per row, one key tile per block) and rows of 1-2 tokens
+    "tiny_blocks": dict(seqlens=[130, 1, 64, 2], block_size=64, n_heads=2, n_groups=1, head_dim=64, head_block=2,
+                        qkv_scale=0.5),
     # scores spread over +-60 in the base-2 domain: later tiles keep exceeding the running reference
     # maximum by far more than the kernel's fast path tolerates, so its redo branch is exercised
     "large_scores": dict(seqlens=[2048, 700], block_size=256, n_heads=4, n_groups=2, head_dim=128, head_block=2,
@@ -116,6 +119,7 @@ BWD_CASES = {
     "multimodal": FWD_CASES["multimodal"],
     "multimodal_image_to_self": FWD_CASES["multimodal_image_to_self"],
     "shared_question": FWD_CASES["shared_question"],
+    "tiny_blocks": FWD_CASES["tiny_blocks"],
 }
 
 
