@@ -13,7 +13,11 @@ pytestmark = pytest.mark.gpu
 def test_plain_cpp_host_drives_the_library(gpu):
     from dcp_amd import build
 
-    assert build.HOST_CHECK_BIN.exists(), "run `python -m dcp_amd.build` first (builds the host check too)"
+    if not build.HOST_CHECK_BIN.exists():  # normally built with the library; a few seconds if not
+        try:
+            build.build_abi_host_check(verbose=False)
+        except Exception as e:  # no compiler on this machine
+            pytest.skip(f"tests/abi_host/abi_host_check is not built and cannot be built here: {e}")
     proc = subprocess.run([str(build.HOST_CHECK_BIN)], capture_output=True, text=True, timeout=100)
     print(proc.stdout, proc.stderr, flush=True)
     assert proc.returncode == 0, proc.stderr
