@@ -70,9 +70,10 @@ struct AttnFwdParams {
 };
 
 // Wave priority by phase: the two waves of a SIMD come from different workgroups and drift
-// through the loop independently; the one in a matrix-dense phase gets the issue slot first
-// (measured 2-3 % on the kernel).
-constexpr int kPrioControl = 0, kPrioFused = 1, kPrioDense = 2;
+// through the loop independently.  Both matrix phases outrank the control code between them
+// (2-3 % on the kernel), and the fused phase, whose vector work is the longer chain, outranks
+// the dense one (another 1.5 %; the other way round it was 1.5 % slower).
+constexpr int kPrioControl = 0, kPrioFused = 2, kPrioDense = 1;
 constexpr int kFwdBN = 64;
 constexpr int kFwdThreads = 256;
 // The running maximum of a row is only raised (and O^T rescaled) when the tile's maximum
