@@ -358,7 +358,6 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     // step requests its own tiles once more, into the stage nobody reads any more.
     const int head_next = more ? kv_head * group + hg_next : kv_head * group + hg;
     const int qt_next = more ? __builtin_ctzll(rem) : qt;
-    request_scalars(head_next, qt_next, st ^ 1);
     const uint16_t* q_lds = tiles[2 * st];
     const uint16_t* do_lds = tiles[2 * st + 1];
 
@@ -419,6 +418,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     u32x4 buf[4];
 #pragma unroll
     for (int o = 0; o < AHEAD; ++o) buf[o] = entry(o);
+    // (after the step's first LDS reads are on their way: the requests are inline assembly that
+    // the compiler moves no memory access across)
+    request_scalars(head_next, qt_next, st ^ 1);
     int loads_issued = 0;
     (void)loads_issued;
 #pragma unroll
