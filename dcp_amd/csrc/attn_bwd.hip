@@ -421,8 +421,6 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     // (after the step's first LDS reads are on their way: the requests are inline assembly that
     // the compiler moves no memory access across)
     request_scalars(head_next, qt_next, st ^ 1);
-    int loads_issued = 0;
-    (void)loads_issued;
 #pragma unroll
     for (int o = 0; o < N1; ++o) {
       const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
@@ -479,14 +477,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   wait_loads();     // the last step's (unused) requests have landed: the tile area is about to be reused
   __syncthreads();  // nobody reads the tiles any more
   float* red = reinterpret_cast<float*>(&tiles[0][0]) + w * (16 * DT * 64);
-  {
-    const f32x16* give = qi == 0 ? dk_acc : dv_acc;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) red[(dt * 16 + i) * 64 + lane] = qi == 0 ? dk_acc[dt][i] : dv_acc[dt][i];
-    (void)give;
-  }
+    for (int i = 0; i < 16; ++i) red[(dt * 16 + i) * 64 + lane] = qi == 0 ? dk_acc[dt][i] : dv_acc[dt][i];
   __syncthreads();
   const float* take = reinterpret_cast<const float*>(&tiles[0][0]) + (w ^ 2) * (16 * DT * 64);
   const float out_scale = qi == 0 ? 1.0f : p.scale;
