@@ -15,7 +15,12 @@ Differences that follow from the kernels, not from the interface:
   dKV buffer and no copy pass (reference :954-1035, :1074-1114);
 * attention rows are launched longest-first (a ``row_order`` table built in
   ``prepare``) so that ragged rows balance across the 256 CUs;
-* communication instructions are rejected: this build runs one GPU.
+* communication instructions run over a ``LocalFabric`` (``fabric.py``): the
+  executors of several devices share one GPU and one process, the sender's
+  copy kernel writes into the receiver's staging buffer and signals with a
+  stream event (two passes instead of the reference's pack, all-to-all and
+  unpack, :1583-2074).  Without a fabric they raise: an exchange between
+  GPUs is not part of this build.
 """
 
 from __future__ import annotations
@@ -38,6 +43,7 @@ from dcp_amd.core.instructions import (
     BufferBlock,
     BufferType,
     CommLaunchInstr,
+    CommType,
     CommWaitInstr,
     ExecutionPlan,
     MemcpyInstr,
@@ -90,6 +96,7 @@ class AttentionExecutor(DCPExecutor):
         iteration_idx: Optional[int] = None,
         tp_rank: Optional[int] = None,
         use_cudagraph: bool = False,
+        fabric=None,
     ):
         super().__init__(
             node_id=node_id,
@@ -101,6 +108,9 @@ class AttentionExecutor(DCPExecutor):
             tp_rank=tp_rank,
         )
         self.process_group = process_group
+        self.fabric = fabric
+        self.pending_comm_ops: Dict[str, dict] = {}
+        self._barrier_generation: Dict[int, int] = {}
         self.n_heads_per_block = n_heads_per_block
         self.head_dim = head_dim
         self.main_stream = torch.cuda.Stream()
@@ -159,6 +169,9 @@ class AttentionExecutor(DCPExecutor):
         touches the host."""
         torch.cuda.nvtx.range_push("AttentionExecutor prepare")
         self._args_cache = {}
+        self.pending_comm_ops = {}
+        if self.fabric is not None:
+            self.fabric.forget(self.rank)
         self.execution_plan = self.fw_exec_plan if forward else self.bw_exec_plan
         self.init_buffers(self.execution_plan)
         for instr_index, instr in enumerate(self.execution_plan.instructions):
@@ -183,6 +196,8 @@ class AttentionExecutor(DCPExecutor):
         plan, is_forward = (
             (self.fw_exec_plan, True) if self.mode == "Forward" else (self.bw_exec_plan, False)
         )
+        if any(isinstance(i, (CommLaunchInstr, CommWaitInstr, BarrierInstr)) for i in plan.instructions):
+            raise NotImplementedError("plans that exchange blocks with other devices are not captured into graphs")
         self.cuda_graph = None
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
@@ -199,11 +214,45 @@ class AttentionExecutor(DCPExecutor):
                 self.cuda_graph.replay()
             else:
                 super().execute(execution_plan, is_forward)
+            for stream in self.streams.values():
+                self.main_stream.wait_stream(stream)
         prev_stream.wait_stream(self.main_stream)
         torch.cuda.nvtx.range_pop()
         if is_forward:
             return self.buffers[BufferType.LOCAL_OUT], self.buffers[BufferType.LOCAL_LSE]
         return self.buffers[BufferType.LOCAL_dQ], self.buffers[BufferType.LOCAL_dKV]
+
+    # -- one instruction at a time (several devices' plans run in turns: fabric.execute_together) --
+    def begin(self, execution_plan):
+        self.execution_plan = execution_plan
+        self.init_buffers(execution_plan)
+        self._prev_stream = torch.cuda.current_stream()
+        self.main_stream.wait_stream(self._prev_stream)
+
+    def step(self, instr_index: int):
+        with torch.cuda.stream(self.main_stream):
+            self.instr_index = instr_index
+            self._execute_instruction(self.execution_plan.instructions[instr_index])
+
+    def finish(self):
+        for stream in self.streams.values():
+            self.main_stream.wait_stream(stream)
+        self._prev_stream.wait_stream(self.main_stream)
+
+    def comm_ready(self, key: str) -> bool:
+        """Have all peers this device receives from under ``key`` launched their sends?"""
+        pending = self.pending_comm_ops.get(key)
+        if pending is None:
+            raise RuntimeError(f"CommWaitInstr {key!r} without a CommLaunchInstr before it")
+        return all(self.fabric.posted(peer, self.rank, key) is not None for peer in pending["recv_peers"])
+
+    def barrier_ready(self, instr_index: int) -> bool:
+        if instr_index not in self._barrier_generation:
+            self._barrier_generation[instr_index] = self.fabric.barrier_arrive(self.rank)
+        if not self.fabric.barrier_passed(self._barrier_generation[instr_index]):
+            return False
+        del self._barrier_generation[instr_index]
+        return True
 
     def forward(self, q, kv):
         self.init_forward_input(q, kv)
@@ -585,15 +634,224 @@ def _handle_sum(exec: AttentionExecutor, instr: SumInstr):
 
 
 # ---------------------------------------------------------------------------
-# communication: not part of a one-GPU build
+# CommLaunchInstr / CommWaitInstr / BarrierInstr over a LocalFabric
 # ---------------------------------------------------------------------------
 
+_DATA_KINDS = (torch.int64, torch.int32, torch.int32, torch.int64, torch.int32, torch.int32, torch.int32)
 
-def _reject_comm(exec: AttentionExecutor, instr: BlockInstrBase):
-    raise NotImplementedError(
-        f"{type(instr).__name__}: inter-GPU communication is not available in this build "
-        "(one GPU owns every block of the plan)"
-    )
+
+def _require_fabric(exec: AttentionExecutor, instr: BlockInstrBase):
+    if exec.fabric is None:
+        raise NotImplementedError(
+            f"{type(instr).__name__}: this executor has no fabric.  Blocks are exchanged between executors "
+            "that share one GPU (get_executor(..., fabric=LocalFabric(...))); an exchange between GPUs is "
+            "not part of this build"
+        )
+
+
+def _comm_block(exec: AttentionExecutor, block: BufferBlock):
+    """What a communication op moves for ``block`` (the views of the reference's
+    ``_prepare_comm_launch`` :1617-1640): ``("data", address, numel)`` for a contiguous run of
+    tokens, ``("lse", base address, token offset, head stride, n_tokens)`` for the
+    ``[head block, n_tokens]`` slice of an LSE buffer."""
+    buf = exec.buffers[block.buffer_type]
+    local = block.buffer_type.startswith("Local")
+    if block.buffer_type in _LSE_BUFFER_TYPES:
+        if local:
+            return ("lse", buf.data_ptr(), exec.execution_plan.local_cu_seqlens[block.index], buf.stride(0), block.n_tokens)
+        return ("lse", buf.data_ptr(), block.index * buf.shape[2], buf.stride(0), block.n_tokens)
+    first = exec.execution_plan.local_cu_seqlens[block.index] if local else block.index
+    per_token = int(np.prod(exec.buffer_per_token_shape[block.buffer_type]))
+    return ("data", buf.data_ptr() + first * buf.stride(0) * buf.element_size(), block.n_tokens * per_token)
+
+
+class _CopyTables:
+    """Argument tables of the copy launches that move a list of blocks between their buffers
+    and a staging buffer: one launch per (dtype, block numel) for data blocks, one for LSE
+    blocks."""
+
+    def __init__(self):
+        self.data = defaultdict(lambda: [[] for _ in range(7)])
+        self.lse = [[] for _ in range(7)]
+        self.hb = None
+
+    def add(self, exec: AttentionExecutor, block: BufferBlock, desc, dtype, staging_address: int, to_staging: bool):
+        if desc[0] == "data":
+            cols = self.data[(dtype, exec.buffer_block_strides[block.buffer_type])]
+            src, dst = (desc[1], staging_address) if to_staging else (staging_address, desc[1])
+            for col, v in zip(cols, (src, 0, 1, dst, 0, 1, desc[2])):
+                col.append(v)
+            return
+        _, base, token_offset, head_stride, n_tokens = desc
+        self.hb = exec.buffers[block.buffer_type].shape[0]
+        mine = (base, token_offset, head_stride)
+        theirs = (staging_address, 0, n_tokens)  # [head block, n_tokens], contiguous
+        src, dst = (mine, theirs) if to_staging else (theirs, mine)
+        for col, v in zip(self.lse, (*src, *dst, n_tokens)):
+            col.append(v)
+
+    def freeze(self, exec: AttentionExecutor):
+        data = {key: tuple(_dev(c, k) for c, k in zip(cols, _DATA_KINDS)) for key, cols in self.data.items()}
+        lse = None
+        if self.lse[0]:
+            lse = tuple(_dev(c, k) for c, k in zip(self.lse, _DATA_KINDS)) + (self.hb, max(self.lse[6]))
+        return data, lse
+
+
+def _launch_copies(frozen):
+    data, lse = frozen
+    for (dtype, block_numel), args in data.items():
+        _COPY_FN[dtype](*args, block_numel, 128)
+    if lse is not None:
+        *tables, hb, max_tokens = lse
+        fused_copy_fp32_varlen_lse(*tables, hb, max_tokens, 1)
+
+
+def _block_numel(exec: AttentionExecutor, block: BufferBlock, desc) -> int:
+    if desc[0] == "data":
+        return desc[2]
+    return exec.buffers[block.buffer_type].shape[0] * desc[4]
+
+
+def _comm_stream(exec: AttentionExecutor, name: Optional[str]):
+    if name is None:
+        return torch.cuda.current_stream()
+    return exec.streams[name]
+
+
+def _prepare_comm_launch(exec: AttentionExecutor, instr: CommLaunchInstr):
+    """Receives: one staging buffer per dtype, the peers' segments in rank order and each
+    peer's blocks in op order (the recv buffer of the reference, :1752-1776), registered with
+    the fabric, and the unpack tables.  Sends: only described here; their tables need the
+    receivers' staging addresses, which exist once every device has prepared, so they are
+    built at the first launch."""
+    _require_fabric(exec, instr)
+    if instr.stream is not None and instr.stream not in exec.streams:
+        exec.streams[instr.stream] = torch.cuda.Stream()
+    sends = []  # (peer, dtype, block, desc)
+    recvs = defaultdict(lambda: defaultdict(list))  # dtype -> peer -> [(block, desc)]
+    for op in instr.comm_ops:
+        peer = exec.get_rank(*op.peer)
+        desc = _comm_block(exec, op.buffer_block)
+        dtype = exec.buffers[op.buffer_block.buffer_type].dtype
+        if dtype not in _COPY_FN:
+            raise ValueError(f"Unsupported dtype {dtype}")
+        if desc[0] == "lse" and dtype != torch.float32:
+            raise ValueError(f"Unsupported LSE dtype {dtype}")
+        if op.comm_type == CommType.SEND:
+            sends.append((peer, dtype, op.buffer_block, desc))
+        else:
+            recvs[dtype][peer].append((op.buffer_block, desc))
+    unpack = _CopyTables()
+    staging_buffers = []
+    for dtype, per_peer in recvs.items():
+        segments, total = {}, 0
+        for peer in sorted(per_peer):
+            numels = [_block_numel(exec, block, desc) for block, desc in per_peer[peer]]
+            segments[peer] = (total, numels)
+            total += sum(numels)
+        staging = torch.empty(total, dtype=dtype, device="cuda")
+        staging_buffers.append(staging)
+        exec.fabric.register_staging(exec.rank, instr.key, dtype, staging, segments)
+        for peer in sorted(per_peer):
+            at = segments[peer][0]
+            for (block, desc), numel in zip(per_peer[peer], segments[peer][1]):
+                unpack.add(exec, block, desc, dtype, staging.data_ptr() + at * staging.element_size(), to_staging=False)
+                at += numel
+    exec._args_cache[exec.instr_index] = {
+        "sends": sends,
+        "pack": None,
+        "send_peers": sorted({peer for peer, _, _, _ in sends}),
+        "recv_peers": sorted({peer for per_peer in recvs.values() for peer in per_peer}),
+        "unpack": unpack.freeze(exec),
+        "staging": staging_buffers,
+    }
+
+
+def _resolve_sends(exec: AttentionExecutor, instr: CommLaunchInstr, cache: dict):
+    pack = _CopyTables()
+    at: Dict[Tuple[int, torch.dtype], int] = {}
+    seen: Dict[Tuple[int, torch.dtype], int] = {}
+    for peer, dtype, block, desc in cache["sends"]:
+        staging, offset, numels = exec.fabric.staging_segment(peer, instr.key, dtype, exec.rank)
+        k = (peer, dtype)
+        i = seen.get(k, 0)
+        numel = _block_numel(exec, block, desc)
+        if i >= len(numels) or numels[i] != numel:
+            raise RuntimeError(
+                f"key {instr.key!r}: send {i} of rank {exec.rank} to rank {peer} has {numel} elements, "
+                f"the receiver expects {numels[i] if i < len(numels) else 'no such block'}"
+            )
+        pos = at.get(k, offset)
+        pack.add(exec, block, desc, dtype, staging.data_ptr() + pos * staging.element_size(), to_staging=True)
+        at[k] = pos + numel
+        seen[k] = i + 1
+    for (peer, dtype), n in seen.items():
+        expected = len(exec.fabric.staging_segment(peer, instr.key, dtype, exec.rank)[2])
+        if n != expected:
+            raise RuntimeError(f"key {instr.key!r}: rank {exec.rank} sends {n} blocks to rank {peer}, which expects {expected}")
+    cache["pack"] = pack.freeze(exec)
+
+
+def _handle_comm_launch(exec: AttentionExecutor, instr: CommLaunchInstr):
+    torch.cuda.nvtx.range_push("CommLaunchInstr")
+    _require_fabric(exec, instr)
+    cache = exec._args_cache[exec.instr_index]
+    if cache["pack"] is None:
+        _resolve_sends(exec, instr, cache)
+    issuing = torch.cuda.current_stream()
+    stream = _comm_stream(exec, instr.stream)
+    stream.wait_stream(issuing)  # the blocks to send were produced by what came before on this device
+    with torch.cuda.stream(stream):
+        for peer in cache["send_peers"]:
+            done = exec.fabric.consumed(peer, instr.key)
+            if done is not None:
+                stream.wait_event(done)  # the receiver's last unpack of this staging buffer
+        _launch_copies(cache["pack"])
+        launched = torch.cuda.Event()
+        launched.record(stream)
+        for peer in cache["send_peers"]:
+            exec.fabric.post(exec.rank, peer, instr.key, launched)
+    exec.pending_comm_ops[instr.key] = {"recv_peers": cache["recv_peers"], "unpack": cache["unpack"], "launched": launched}
+    torch.cuda.nvtx.range_pop()
+
+
+def _prepare_comm_wait(exec: AttentionExecutor, instr: CommWaitInstr):
+    _require_fabric(exec, instr)
+    if instr.stream is not None and instr.stream not in exec.streams:
+        exec.streams[instr.stream] = torch.cuda.Stream()
+
+
+def _handle_comm_wait(exec: AttentionExecutor, instr: CommWaitInstr):
+    torch.cuda.nvtx.range_push("CommWaitInstr")
+    _require_fabric(exec, instr)
+    if not exec.comm_ready(instr.key):
+        raise RuntimeError(
+            f"CommWaitInstr {instr.key!r} on rank {exec.rank}: a peer has not launched its sends yet "
+            "(run the devices' plans with fabric.execute_together)"
+        )
+    pending = exec.pending_comm_ops.pop(instr.key)
+    stream = _comm_stream(exec, instr.stream)
+    with torch.cuda.stream(stream):
+        # the wait covers this device's own part of the exchange too, as waiting for the
+        # reference's all-to-all does: what the launch's stream did before it is done
+        stream.wait_event(pending["launched"])
+        for peer in pending["recv_peers"]:
+            stream.wait_event(exec.fabric.take(peer, exec.rank, instr.key))
+        _launch_copies(pending["unpack"])
+        if pending["recv_peers"]:
+            event = torch.cuda.Event()
+            event.record(stream)
+            exec.fabric.set_consumed(exec.rank, instr.key, event)
+    torch.cuda.nvtx.range_pop()
+
+
+def _handle_barrier(exec: AttentionExecutor, instr: BarrierInstr):
+    """All devices have reached the barrier when this runs (``execute_together`` holds a device
+    back until then): what is left of the reference's all-reduce (:2006-2012) is to wait for
+    the device's own work."""
+    _require_fabric(exec, instr)
+    torch.cuda.current_stream().synchronize()
 
 
 def get_executor(
@@ -610,15 +868,22 @@ def get_executor(
     iteration_idx: Optional[int] = None,
     tp_rank: Optional[int] = None,
     use_cudagraph: bool = False,
+    fabric=None,
 ):
-    """Factory with the reference's signature (:2077-2133).  ``exec_context``
-    only supplies ``n_devices_per_node`` / ``n_nodes`` and may be ``None``."""
+    """Factory with the reference's signature (:2077-2133) plus ``fabric``.  ``exec_context``
+    only supplies ``n_devices_per_node`` / ``n_nodes`` and may be ``None``.  With a
+    ``LocalFabric`` the executor is one of several devices sharing this GPU: the fabric gives
+    the device grid and the plan says which device it is."""
     if executor_impl != "python":
         raise ValueError(f"Unsupported executor_impl: {executor_impl}")
     n_devices_per_node = getattr(exec_context, "n_devices_per_node", 1)
     n_nodes = getattr(exec_context, "n_nodes", 1)
     rank = 0
-    if torch.distributed.is_available() and torch.distributed.is_initialized():
+    if fabric is not None:
+        plan = fw_exec_plan if fw_exec_plan is not None else bw_exec_plan
+        n_devices_per_node, n_nodes = fabric.n_devices_per_node, fabric.n_nodes
+        rank = plan.node_id * n_devices_per_node + plan.local_device_id
+    elif torch.distributed.is_available() and torch.distributed.is_initialized():
         rank = torch.distributed.get_rank(group=process_group)
     executor = AttentionExecutor(
         fw_exec_plan=fw_exec_plan,
@@ -636,19 +901,22 @@ def get_executor(
         iteration_idx=iteration_idx,
         tp_rank=tp_rank,
         use_cudagraph=use_cudagraph,
+        fabric=fabric,
     )
     executor.register_handler(MemcpyInstr, _handle_memcpy)
     executor.register_handler(AttnInstr, _handle_attn)
     executor.register_handler(AttnBackwardInstr, _handle_attn_bw)
     executor.register_handler(AttnReductionInstr, _handle_reduction)
     executor.register_handler(SumInstr, _handle_sum)
-    executor.register_handler(CommLaunchInstr, _reject_comm)
-    executor.register_handler(CommWaitInstr, _reject_comm)
-    executor.register_handler(BarrierInstr, _reject_comm)
+    executor.register_handler(CommLaunchInstr, _handle_comm_launch)
+    executor.register_handler(CommWaitInstr, _handle_comm_wait)
+    executor.register_handler(BarrierInstr, _handle_barrier)
     executor.register_prep_handler(MemcpyInstr, _prepare_memcpy)
     executor.register_prep_handler(AttnInstr, _prepare_attn)
     executor.register_prep_handler(AttnBackwardInstr, _prepare_attn_bw)
     executor.register_prep_handler(AttnReductionInstr, _prepare_reduction)
     executor.register_prep_handler(SumInstr, _prepare_sum)
+    executor.register_prep_handler(CommLaunchInstr, _prepare_comm_launch)
+    executor.register_prep_handler(CommWaitInstr, _prepare_comm_wait)
     executor.check_all_handlers_registered()
     return executor

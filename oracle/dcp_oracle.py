@@ -23,7 +23,9 @@ repository root):
                           LSE = logsumexp, out=0 / lse=+inf for empty rows) is
                           restated here
   run_plan                instruction semantics of
-                          dcp/runtime/flash_attention/executor.py:606-1546
+                          dcp/runtime/flash_attention/executor.py:606-1546;
+                          block exchange between devices (CommLaunchInstr /
+                          CommWaitInstr) executor.py:1583-2074
 
 Pinning (tests/test_oracle.py): block movement against numpy fancy indexing
 and gather/scatter round trips; merge against scipy.special.logsumexp, the
@@ -252,6 +254,46 @@ class PlanOracle:
             getattr(self, "_" + type(instr).__name__)(instr)
         return self.buffers
 
+    # -- communication (several devices' plans run together, see run_plans_together) ----------
+    def attach(self, mailbox: dict, rank: int, n_devices_per_node: int) -> None:
+        self.mailbox, self.rank, self.n_devices_per_node = mailbox, rank, n_devices_per_node
+        self.expected: Dict[str, list] = {}
+
+    def _block_view(self, block):
+        """The elements a communication op moves for ``block``: the same views as
+        _prepare_comm_launch builds (executor.py:1617-1640)."""
+        buf, n = self.buffers[block.buffer_type], block.n_tokens
+        if block.buffer_type.startswith("Local"):
+            off = self.plan.local_cu_seqlens[block.index]
+            return buf[:, off : off + n] if block.buffer_type in _LSE_TYPES else buf[off : off + n]
+        return buf[:, block.index, :n] if block.buffer_type in _LSE_TYPES else buf[block.index, :n]
+
+    def _CommLaunchInstr(self, instr):
+        """Sends are snapshotted at launch, in op order per peer (the send buffer of
+        executor.py:1949-1976); receives land at the matching wait (:2043-2073)."""
+        recvs = []
+        for op in instr.comm_ops:
+            peer = op.peer[0] * self.n_devices_per_node + op.peer[1]
+            if op.comm_type == 0:  # CommType.SEND
+                self.mailbox.setdefault((self.rank, peer, instr.key), []).append(self._block_view(op.buffer_block).copy())
+            else:
+                recvs.append((peer, op.buffer_block))
+        self.expected[instr.key] = recvs
+
+    def comm_ready(self, key: str) -> bool:
+        need: Dict[int, int] = {}
+        for peer, _ in self.expected[key]:
+            need[peer] = need.get(peer, 0) + 1
+        return all(len(self.mailbox.get((peer, self.rank, key), [])) >= n for peer, n in need.items())
+
+    def _CommWaitInstr(self, instr):
+        assert self.comm_ready(instr.key), "wait before the peers' launches"
+        for peer, block in self.expected.pop(instr.key):
+            data = self.mailbox[(peer, self.rank, instr.key)].pop(0)
+            view = self._block_view(block)
+            assert view.shape == data.shape, (view.shape, data.shape)
+            view[...] = data
+
     # -- instructions --------------------------------------------------------
     def _MemcpyInstr(self, instr):
         cu = self.plan.local_cu_seqlens
@@ -327,6 +369,30 @@ class PlanOracle:
                 self._store(d.buffer_type, slice(off, off + n), total)
             else:
                 self._store(d.buffer_type, (d.index, slice(0, n)), total)
+
+
+def run_plans_together(oracles: Sequence["PlanOracle"], n_devices_per_node: int) -> None:
+    """Runs the plans of several devices (``oracles[rank]``) to the end, each as far as its
+    next wait whose peers have not launched yet, in turns: a device's sends are visible to its
+    peers from its CommLaunchInstr on, as with the asynchronous all-to-all of
+    executor.py:1977-1999."""
+    mailbox: dict = {}
+    for rank, o in enumerate(oracles):
+        o.attach(mailbox, rank, n_devices_per_node)
+    cursor = [0] * len(oracles)
+    while any(c < len(o.plan.instructions) for c, o in zip(cursor, oracles)):
+        progressed = False
+        for rank, o in enumerate(oracles):
+            instrs = o.plan.instructions
+            while cursor[rank] < len(instrs):
+                instr = instrs[cursor[rank]]
+                if type(instr).__name__ == "CommWaitInstr" and not o.comm_ready(instr.key):
+                    break
+                getattr(o, "_" + type(instr).__name__)(instr)
+                cursor[rank] += 1
+                progressed = True
+        assert progressed, "the plans wait for each other"
+    assert all(len(v) == 0 for v in mailbox.values()), "blocks sent but never received"
 
 
 # ---------------------------------------------------------------------------

@@ -81,9 +81,98 @@ def run_plan_oracle(case, backward=False):
         pb.set("LocalKV", layout.to_local_kv(case["kv"]).float().numpy())
         pb.set("LocalOut", bufs["LocalOut"])
         pb.buffers["LocalLSE"][...] = bufs["LocalLSE"]
-        pb.set("LocalOut", bufs["LocalOut"])
         pb.set("LocaldOut", layout.to_local_q(case["dout"]).float().numpy())
         b2 = pb.run()
         res += [layout.from_local_q(torch.from_numpy(b2["LocaldQ"].copy())),
                 layout.from_local_kv(torch.from_numpy(b2["LocaldKV"].copy()))]
     return res
+
+
+# ---------------------------------------------------------------------------
+# several devices (their executors share the one GPU; blocks travel over a LocalFabric)
+# ---------------------------------------------------------------------------
+
+
+def make_multi_case(n_nodes, n_devices_per_node, seqlens, block_size, n_heads, n_groups, head_dim, head_block,
+                    mask="causal", mask_info=None, dtype="bf16", seed=0, mask_kwargs=None):
+    from dcp_amd.runtime.flash_attention.multi_device import build_multi_device_plans
+
+    mask_t = MASK_FNS[mask](list(seqlens), list(seqlens), torch.int32, mask_info, **(mask_kwargs or {}))
+    fw, bw, layouts = build_multi_device_plans(n_nodes, n_devices_per_node, seqlens, block_size, n_heads, n_groups,
+                                               head_dim, head_block, mask_t, dtype=TORCH_DTYPE[dtype])
+    g = torch.Generator().manual_seed(seed)
+    T = sum(seqlens)
+    q = torch.randn(T, n_heads, head_dim, generator=g).to(TORCH_DTYPE[dtype])
+    kv = torch.randn(T, 2, n_groups, head_dim, generator=g).to(TORCH_DTYPE[dtype])
+    dout = torch.randn(T, n_heads, head_dim, generator=g).to(TORCH_DTYPE[dtype])
+    return dict(fw=fw, bw=bw, layouts=layouts, mask=mask_t, q=q, kv=kv, dout=dout, seqlens=list(seqlens),
+                head_block=head_block, head_dim=head_dim, dtype=dtype, n_nodes=n_nodes,
+                n_devices_per_node=n_devices_per_node)
+
+
+def _sum_over_ranks(parts):
+    total = parts[0].clone()
+    for p in parts[1:]:
+        total += p
+    return total
+
+
+def run_multi_oracle(case, backward=False):
+    """All devices' plans on the numpy oracle.  Global-layout (out, lse[, dq, dkv])."""
+    lays = case["layouts"]
+    fw = [oracle.PlanOracle(p, case["head_block"], case["head_dim"]) for p in case["fw"]]
+    for o, lay in zip(fw, lays):
+        o.set("LocalQ", lay.to_local_q(case["q"]).float().numpy())
+        o.set("LocalKV", lay.to_local_kv(case["kv"]).float().numpy())
+    oracle.run_plans_together(fw, case["n_devices_per_node"])
+    outs = [torch.from_numpy(o.buffers["LocalOut"].copy()) for o in fw]
+    lses = [torch.from_numpy(o.buffers["LocalLSE"].copy()) for o in fw]
+    res = [_sum_over_ranks([lay.from_local_q(x) for lay, x in zip(lays, outs)]),
+           _sum_over_ranks([lay.from_local_lse(x) for lay, x in zip(lays, lses)])]
+    if backward:
+        bw = [oracle.PlanOracle(p, case["head_block"], case["head_dim"]) for p in case["bw"]]
+        for o, f, lay in zip(bw, fw, lays):
+            o.set("LocalQ", lay.to_local_q(case["q"]).float().numpy())
+            o.set("LocalKV", lay.to_local_kv(case["kv"]).float().numpy())
+            o.set("LocalOut", f.buffers["LocalOut"])
+            o.buffers["LocalLSE"][...] = f.buffers["LocalLSE"]
+            o.set("LocaldOut", lay.to_local_q(case["dout"]).float().numpy())
+        oracle.run_plans_together(bw, case["n_devices_per_node"])
+        res += [_sum_over_ranks([lay.from_local_q(torch.from_numpy(o.buffers["LocaldQ"].copy())) for lay, o in zip(lays, bw)]),
+                _sum_over_ranks([lay.from_local_kv(torch.from_numpy(o.buffers["LocaldKV"].copy())) for lay, o in zip(lays, bw)])]
+    return res
+
+
+def run_multi_executor(case, backward=False, repeats=1):
+    """All devices' plans through HIP executors that share the GPU and one LocalFabric."""
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric, execute_together
+
+    fabric = LocalFabric(case["n_nodes"], case["n_devices_per_node"])
+    lays = case["layouts"]
+    exs = [get_executor(case["head_block"], case["head_dim"], None, fw_exec_plan=f, bw_exec_plan=b, fabric=fabric)
+           for f, b in zip(case["fw"], case["bw"])]
+    for ex in exs:
+        ex.prepare(forward=True)
+    for ex, lay in zip(exs, lays):
+        ex.init_forward_input(lay.to_local_q(case["q"]).cuda(), lay.to_local_kv(case["kv"]).cuda())
+    for _ in range(repeats):
+        execute_together(exs, forward=True)
+    torch.cuda.synchronize()
+    outs = [ex.buffers["LocalOut"].clone() for ex in exs]
+    lses = [ex.buffers["LocalLSE"].clone() for ex in exs]
+    res = [_sum_over_ranks([lay.from_local_q(x.cpu()) for lay, x in zip(lays, outs)]),
+           _sum_over_ranks([lay.from_local_lse(x.cpu()) for lay, x in zip(lays, lses)])]
+    if backward:
+        for ex in exs:
+            ex.switch_to_backward()
+        for ex, lay, o, l in zip(exs, lays, outs, lses):
+            ex.set_local_out_lse(o, l)
+            ex.init_forward_input(lay.to_local_q(case["q"]).cuda(), lay.to_local_kv(case["kv"]).cuda())
+            ex.init_backward_input(lay.to_local_q(case["dout"]).cuda())
+        for _ in range(repeats):
+            execute_together(exs, forward=False)
+        torch.cuda.synchronize()
+        res += [_sum_over_ranks([lay.from_local_q(ex.buffers["LocaldQ"].cpu()) for lay, ex in zip(lays, exs)]),
+                _sum_over_ranks([lay.from_local_kv(ex.buffers["LocaldKV"].cpu()) for lay, ex in zip(lays, exs)])]
+    return res, exs
