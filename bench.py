@@ -306,6 +306,65 @@ def movement_microbench(iters=5, bs=512):
     )
 
 
+def exchange_microbench(n_devices=4, blocks_per_pair=64, bs=1024, hb=4, d=128, iters=5):
+    """Block exchange between devices' executors that share the GPU (LocalFabric): every device
+    sends ``blocks_per_pair`` Q blocks of [bs, hb, d] bf16 (1 MiB at the defaults) to every other
+    device; the sender's copy writes into the receiver's staging buffer, the receiver unpacks
+    into its slots.  Each block is read and written once per pass, two passes."""
+    import torch
+    from dcp_amd.core.instructions import (BufferBlock, BufferInfo, BufferType, CommLaunchInstr, CommOp,
+                                            CommType, CommWaitInstr, DType, ExecutionPlan)
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric, execute_together
+
+    n_send = blocks_per_pair * (n_devices - 1)
+    numel = bs * hb * d
+    info = {
+        BufferType.LOCAL_Q: BufferInfo(n_send, bs, numel, DType.BFLOAT16, (n_send * bs, hb, d), (hb, d)),
+        BufferType.BUFFER_Q: BufferInfo(n_send, bs, numel, DType.BFLOAT16, (n_send, bs, hb, d), (hb, d)),
+    }
+    cu = [i * bs for i in range(n_send + 1)]
+    plans = []
+    for r in range(n_devices):
+        peers = [p for p in range(n_devices) if p != r]
+        ops = []
+        for k, p in enumerate(peers):
+            for i in range(blocks_per_pair):
+                ops.append(CommOp(CommType.SEND, (0, p), BufferBlock(BufferType.LOCAL_Q, k * blocks_per_pair + i, bs)))
+                ops.append(CommOp(CommType.RECV, (0, p), BufferBlock(BufferType.BUFFER_Q, k * blocks_per_pair + i, bs)))
+        plans.append(ExecutionPlan([CommLaunchInstr("S0", ops), CommWaitInstr("S0")], 1, n_devices, 0, r, 1, cu, info))
+    fabric = LocalFabric(1, n_devices)
+    exs = [get_executor(hb, d, None, fw_exec_plan=p, fabric=fabric) for p in plans]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    for ex in exs:
+        ex.prepare(forward=True)
+        ex.buffers[BufferType.LOCAL_Q].copy_(torch.randn(n_send * bs, hb, d, device="cuda", generator=g))
+    execute_together(exs)
+    torch.cuda.synchronize()
+    exact = True
+    for r, ex in enumerate(exs):  # slot k*bpp+i of r came from peer p's block (index of r among p's peers)*bpp+i
+        for k, p in enumerate([p for p in range(n_devices) if p != r]):
+            kp = [q for q in range(n_devices) if q != p].index(r)
+            got = ex.buffers[BufferType.BUFFER_Q][k * blocks_per_pair : (k + 1) * blocks_per_pair]
+            want = exs[p].buffers[BufferType.LOCAL_Q][kp * blocks_per_pair * bs : (kp + 1) * blocks_per_pair * bs]
+            exact &= bool(torch.equal(got.reshape(-1), want.reshape(-1)))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        execute_together(exs)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / iters
+    moved = n_devices * n_send * numel * 2  # bytes that change device per exchange
+    return dict(
+        workload=f"{n_devices} devices' executors on one GPU, {blocks_per_pair} blocks of {numel * 2 >> 10} KiB to every peer",
+        ms_per_exchange=round(ms, 3),
+        moved_GB_per_exchange=round(moved / 1e9, 3),
+        hbm_GBps=round(4 * moved / (ms * 1e-3) / 1e9, 1),  # pack + unpack, each a read and a write
+        bit_exact=exact,
+    )
+
+
 # ---------------------------------------------------------------------------
 # CPU baseline: the oracle on a bounded, seeded sample of q-block rows
 # ---------------------------------------------------------------------------
@@ -483,6 +542,8 @@ def main():
         del ex_f, ex_b
         torch.cuda.empty_cache()
         extra["block_movement"] = movement_microbench()
+        torch.cuda.empty_cache()
+        extra["block_exchange"] = exchange_microbench()
     if not args.no_cpu:
         extra["stage_packer"] = stage_packer_timing()
 
