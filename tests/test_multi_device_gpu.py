@@ -93,3 +93,85 @@ def test_comm_without_fabric_raises():
     ex = get_executor(case["head_block"], case["head_dim"], None, fw_exec_plan=case["fw"][0], bw_exec_plan=case["bw"][0])
     with pytest.raises(NotImplementedError, match="fabric"):
         ex.prepare(forward=True)
+
+
+def test_two_phase_relay_on_a_side_stream_and_barrier():
+    """Device 0 sends blocks to device 1 (key S1); device 1 waits for them on its second-phase
+    stream and forwards them to device 2 from there (key S1P2), the shape of the reference's
+    inter-node then intra-node relay (dcp/core/scheduler.py:1001-1048).  A barrier follows."""
+    from dcp_amd.core.instructions import (BarrierInstr, BufferBlock, BufferInfo, BufferType, CommLaunchInstr, CommOp,
+                                            CommType, CommWaitInstr, DType, ExecutionPlan)
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric, execute_together
+
+    print("multi-device two-phase relay", flush=True)
+    n, bs, hb, d = 6, 128, 2, 64
+    tokens = [bs, 37, bs, 5, 100, bs]  # ragged blocks
+    numel = bs * hb * d
+    cu = [0]
+    for t in tokens:
+        cu.append(cu[-1] + t)
+    info = {
+        BufferType.LOCAL_Q: BufferInfo(n, bs, numel, DType.BFLOAT16, (cu[-1], hb, d), (hb, d)),
+        BufferType.BUFFER_Q: BufferInfo(n, bs, numel, DType.BFLOAT16, (n, bs, hb, d), (hb, d)),
+        BufferType.LOCAL_LSE: BufferInfo(n, bs, bs * hb, DType.FLOAT32, (hb, cu[-1]), (1,)),
+        BufferType.BUFFER_LSE: BufferInfo(n, bs, bs * hb, DType.FLOAT32, (hb, n, bs), (1,)),
+    }
+
+    def ops(kind, peer, local):
+        out = []
+        for i, t in enumerate(tokens):
+            q = BufferBlock(BufferType.LOCAL_Q if local else BufferType.BUFFER_Q, i if local else n - 1 - i, t)
+            l = BufferBlock(BufferType.LOCAL_LSE if local else BufferType.BUFFER_LSE, i if local else n - 1 - i, t)
+            out += [CommOp(kind, peer, q), CommOp(kind, peer, l)]
+        return out
+
+    plans = [
+        [CommLaunchInstr("S1", ops(CommType.SEND, (0, 1), True)), CommWaitInstr("S1"), BarrierInstr()],
+        [CommLaunchInstr("S1", ops(CommType.RECV, (0, 0), False)), CommWaitInstr("S1", stream="second_phase"),
+         CommLaunchInstr("S1P2", ops(CommType.SEND, (0, 2), False), stream="second_phase"), CommWaitInstr("S1P2"),
+         BarrierInstr()],
+        [CommLaunchInstr("S1P2", ops(CommType.RECV, (0, 1), False), stream="second_phase"), CommWaitInstr("S1P2"),
+         BarrierInstr()],
+    ]
+    fabric = LocalFabric(1, 3)
+    exs = [get_executor(hb, d, None, fw_exec_plan=ExecutionPlan(p, 1, 3, 0, r, 1, cu, info), fabric=fabric)
+           for r, p in enumerate(plans)]
+    g = torch.Generator().manual_seed(3)
+    src_q = torch.randn(cu[-1], hb, d, generator=g).to(torch.bfloat16)
+    src_l = torch.randn(hb, cu[-1], generator=g)
+    for ex in exs:
+        ex.prepare(forward=True)
+    exs[0].buffers[BufferType.LOCAL_Q].copy_(src_q)
+    exs[0].buffers[BufferType.LOCAL_LSE].copy_(src_l)
+    for _ in range(2):
+        execute_together(exs)
+    torch.cuda.synchronize()
+    for ex in exs[1:]:
+        for i, t in enumerate(tokens):
+            slot = n - 1 - i
+            assert torch.equal(ex.buffers[BufferType.BUFFER_Q][slot, :t].cpu(), src_q[cu[i] : cu[i] + t])
+            assert torch.equal(ex.buffers[BufferType.BUFFER_LSE][:, slot, :t].cpu(), src_l[:, cu[i] : cu[i] + t])
+            assert not ex.buffers[BufferType.BUFFER_Q][slot, t:].any()  # padding rows untouched
+
+
+def test_mismatched_exchange_is_rejected():
+    """A send the receiver has no matching receive for fails at the launch, before any kernel."""
+    from dcp_amd.core.instructions import (BufferBlock, BufferInfo, BufferType, CommLaunchInstr, CommOp, CommType,
+                                            CommWaitInstr, DType, ExecutionPlan)
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric, execute_together
+
+    bs, hb, d = 64, 1, 64
+    info = {BufferType.LOCAL_Q: BufferInfo(2, bs, bs * hb * d, DType.BFLOAT16, (2 * bs, hb, d), (hb, d)),
+            BufferType.BUFFER_Q: BufferInfo(2, bs, bs * hb * d, DType.BFLOAT16, (2, bs, hb, d), (hb, d))}
+    send = [CommOp(CommType.SEND, (0, 1), BufferBlock(BufferType.LOCAL_Q, i, bs)) for i in range(2)]
+    recv = [CommOp(CommType.RECV, (0, 0), BufferBlock(BufferType.BUFFER_Q, 0, bs - 1))]  # one block, wrong size
+    plans = [[CommLaunchInstr("S0", send), CommWaitInstr("S0")], [CommLaunchInstr("S0", recv), CommWaitInstr("S0")]]
+    fabric = LocalFabric(1, 2)
+    exs = [get_executor(hb, d, None, fw_exec_plan=ExecutionPlan(p, 1, 2, 0, r, 1, [0, bs, 2 * bs], info), fabric=fabric)
+           for r, p in enumerate(plans)]
+    for ex in exs:
+        ex.prepare(forward=True)
+    with pytest.raises(RuntimeError, match="receiver expects"):
+        execute_together(exs)
