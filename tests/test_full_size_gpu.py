@@ -3,7 +3,8 @@ and seeded samples of the oracle (the full oracle would take hours):
 
 * config 2 (Llama-3-8B shape, 65536 tokens, causal, bs 1024, GQA 32/8):
   sampled (sequence, head) parity against dense fp64 attention, exact
-  linearity of the backward in dO, bit-reproducibility, HIP-graph replays;
+  linearity of the backward in dO, bit-reproducibility, HIP-graph replays; the same schedule
+  placed on four devices whose executors share the GPU reproduces the one-device result;
 * config 3 (lambda mask, sink 64 + window 4096) at 32768 tokens: sampled parity against the
   oracle; at the full 131072 tokens and config 4 (shared prefix, 98304 tokens, 40/8 heads,
   bs 512, every row's kv blocks in two partials) a whole (sequence, kv head) group is checked
@@ -188,6 +189,55 @@ def test_config2_hip_graph_replays_match_eager(gpu):
     ex.cuda_graph = None
     ref2, _ = ex.forward(q2, kv)
     assert torch.equal(out2, ref2)
+
+
+def test_config2_split_over_four_devices_matches_one_device(gpu):
+    """The 65536-token schedule placed on four devices (their executors share the GPU and
+    exchange Q/KV blocks, partial outputs and partial gradients over a LocalFabric) gives what one
+    device owning every block gives, up to the extra roundings of partials that travel in bf16."""
+    from dcp_amd.core.instructions import BufferType as B
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric, execute_together
+    from dcp_amd.runtime.flash_attention.multi_device import build_multi_device_plans
+
+    wl = bench.workload("llama3_8b_causal_64k")
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl)
+    one = dict(q=layout.from_local_q(t[B.LOCAL_Q]), kv=layout.from_local_kv(t[B.LOCAL_KV]),
+               out=layout.from_local_q(t[B.LOCAL_OUT]), lse=layout.from_local_lse(t[B.LOCAL_LSE]),
+               dout=layout.from_local_q(t[B.LOCAL_dOUT]), dq=layout.from_local_q(t[B.LOCAL_dQ]),
+               dkv=layout.from_local_kv(t[B.LOCAL_dKV]))
+    del ex_f, ex_b, t
+    torch.cuda.empty_cache()
+    fws, bws, lays = build_multi_device_plans(1, 4, wl["seqlens"], wl["block_size"], wl["n_heads"], wl["n_groups"],
+                                              wl["head_dim"], wl["head_block"], mask, dtype=torch.bfloat16)
+    fabric = LocalFabric(1, 4)
+    exs = [get_executor(wl["head_block"], wl["head_dim"], None, fw_exec_plan=f, bw_exec_plan=b, fabric=fabric)
+           for f, b in zip(fws, bws)]
+    print("four devices: forward", flush=True)
+    for ex, lay in zip(exs, lays):
+        ex.prepare(forward=True)
+        ex.init_forward_input(lay.to_local_q(one["q"]), lay.to_local_kv(one["kv"]))
+    execute_together(exs, forward=True)
+    torch.cuda.synchronize()
+    outs = [ex.buffers[B.LOCAL_OUT].clone() for ex in exs]
+    lses = [ex.buffers[B.LOCAL_LSE].clone() for ex in exs]
+    out = sum(lay.from_local_q(x) for lay, x in zip(lays, outs))
+    lse = sum(lay.from_local_lse(x) for lay, x in zip(lays, lses))
+    assert float((out.float() - one["out"].float()).abs().max()) <= 2e-2
+    assert float((lse - one["lse"]).abs().max()) <= 1e-3
+    print("four devices: backward", flush=True)
+    for ex, lay, o, l in zip(exs, lays, outs, lses):
+        ex.switch_to_backward()
+        ex.set_local_out_lse(o, l)
+        ex.init_forward_input(lay.to_local_q(one["q"]), lay.to_local_kv(one["kv"]))
+        ex.init_backward_input(lay.to_local_q(one["dout"]))
+    execute_together(exs, forward=False)
+    torch.cuda.synchronize()
+    dq = sum(lay.from_local_q(ex.buffers[B.LOCAL_dQ]) for lay, ex in zip(lays, exs))
+    dkv = sum(lay.from_local_kv(ex.buffers[B.LOCAL_dKV]) for lay, ex in zip(lays, exs))
+    for got, want in ((dq, one["dq"]), (dkv, one["dkv"])):
+        err = (got.float() - want.float()).abs()
+        assert bool((err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * float(want.float().abs().max())).all())
 
 
 def test_config3_lambda_mask_sampled_parity(gpu):
