@@ -61,3 +61,88 @@ def test_plans_with_exchange_survive_the_wire_format():
     for plan in case["fw"] + case["bw"]:
         restored, rest = ExecutionPlan.deserialize(plan.serialize())
         assert restored == plan and rest == b""
+
+
+# ---------------------------------------------------------------------------
+# the fabric's host logic, with stand-in executors (no GPU)
+# ---------------------------------------------------------------------------
+
+
+class _StubExecutor:
+    """Has the stepping interface of AttentionExecutor; 'launch' posts a token to the fabric,
+    'wait' needs the tokens of the peers it names."""
+
+    def __init__(self, fabric, rank, instrs, recv_from):
+        from dcp_amd.core.instructions import ExecutionPlan
+
+        self.fabric, self.rank, self.recv_from, self.log = fabric, rank, recv_from, []
+        self.fw_exec_plan = self.bw_exec_plan = ExecutionPlan(instrs, 1, fabric.n_ranks, 0, rank, 1, [0], {})
+        self._arrived = {}
+
+    def begin(self, plan):
+        self.plan = plan
+
+    def finish(self):
+        self.log.append("finish")
+
+    def comm_ready(self, key):
+        return all(self.fabric.posted(p, self.rank, key) is not None for p in self.recv_from.get(key, []))
+
+    def barrier_ready(self, index):
+        if index not in self._arrived:
+            self._arrived[index] = self.fabric.barrier_arrive(self.rank)
+        return self.fabric.barrier_passed(self._arrived[index])
+
+    def step(self, index):
+        instr = self.plan.instructions[index]
+        self.log.append(type(instr).__name__ + ":" + getattr(instr, "key", ""))
+        if isinstance(instr, CommLaunchInstr):
+            for peer in range(self.fabric.n_ranks):
+                if peer != self.rank:
+                    self.fabric.post(self.rank, peer, instr.key, object())
+        elif isinstance(instr, CommWaitInstr):
+            for p in self.recv_from.get(instr.key, []):
+                self.fabric.take(p, self.rank, instr.key)
+
+
+def test_execute_together_interleaves_devices_and_detects_cycles():
+    from dcp_amd.core.instructions import BarrierInstr
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric, execute_together
+
+    fabric = LocalFabric(1, 2)
+    # device 0 waits for device 1 before it launches anything device 1 could wait for, and
+    # device 1 launches first: runs through
+    a = _StubExecutor(fabric, 0, [CommWaitInstr("A"), CommLaunchInstr("B", []), BarrierInstr()], {"A": [1]})
+    b = _StubExecutor(fabric, 1, [CommLaunchInstr("A", []), CommWaitInstr("B"), BarrierInstr()], {"B": [0]})
+    execute_together([a, b])
+    assert a.log == ["CommWaitInstr:A", "CommLaunchInstr:B", "BarrierInstr:", "finish"]
+    assert b.log == ["CommLaunchInstr:A", "CommWaitInstr:B", "BarrierInstr:", "finish"]
+    # both wait first: nobody can run
+    fabric = LocalFabric(1, 2)
+    a = _StubExecutor(fabric, 0, [CommWaitInstr("A"), CommLaunchInstr("B", [])], {"A": [1]})
+    b = _StubExecutor(fabric, 1, [CommWaitInstr("B"), CommLaunchInstr("A", [])], {"B": [0]})
+    with pytest.raises(RuntimeError, match="wait for each other"):
+        execute_together([a, b])
+    # a barrier one device never reaches
+    fabric = LocalFabric(1, 2)
+    a = _StubExecutor(fabric, 0, [BarrierInstr()], {})
+    b = _StubExecutor(fabric, 1, [], {})
+    with pytest.raises(RuntimeError, match="wait for each other"):
+        execute_together([a, b])
+
+
+def test_fabric_staging_registry():
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric
+
+    fabric = LocalFabric(2, 2)
+    assert fabric.n_ranks == 4
+    staging = object()
+    fabric.register_staging(3, "S0", torch.bfloat16, staging, {1: (0, [8, 8]), 2: (16, [4])})
+    assert fabric.staging_segment(3, "S0", torch.bfloat16, 2) == (staging, 16, [4])
+    with pytest.raises(RuntimeError, match="no matching receives"):
+        fabric.staging_segment(3, "S0", torch.bfloat16, 0)
+    with pytest.raises(RuntimeError, match="no matching receives"):
+        fabric.staging_segment(3, "S0", torch.float32, 1)
+    fabric.forget(3)
+    with pytest.raises(RuntimeError, match="no matching receives"):
+        fabric.staging_segment(3, "S0", torch.bfloat16, 1)
