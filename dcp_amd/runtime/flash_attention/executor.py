@@ -761,6 +761,7 @@ def _prepare_comm_launch(exec: AttentionExecutor, instr: CommLaunchInstr):
     exec._args_cache[exec.instr_index] = {
         "sends": sends,
         "pack": None,
+        "epoch": None,
         "send_peers": sorted({peer for peer, _, _, _ in sends}),
         "recv_peers": sorted({peer for per_peer in recvs.values() for peer in per_peer}),
         "unpack": unpack.freeze(exec),
@@ -797,8 +798,10 @@ def _handle_comm_launch(exec: AttentionExecutor, instr: CommLaunchInstr):
     torch.cuda.nvtx.range_push("CommLaunchInstr")
     _require_fabric(exec, instr)
     cache = exec._args_cache[exec.instr_index]
-    if cache["pack"] is None:
+    if cache["pack"] is None or cache["epoch"] != exec.fabric.epoch:
+        # first launch, or a peer has prepared again since: its staging buffers are new ones
         _resolve_sends(exec, instr, cache)
+        cache["epoch"] = exec.fabric.epoch
     issuing = torch.cuda.current_stream()
     stream = _comm_stream(exec, instr.stream)
     stream.wait_stream(issuing)  # the blocks to send were produced by what came before on this device

@@ -36,11 +36,13 @@ class LocalFabric:
         self._posted: Dict[Tuple[int, int, str], torch.cuda.Event] = {}
         self._consumed: Dict[Tuple[int, str], torch.cuda.Event] = {}
         self._barrier_arrivals = [0] * self.n_ranks
+        self.epoch = 0  # changes whenever a staging buffer is (re)registered or dropped
 
     # -- prepare time ----------------------------------------------------------------------
     def register_staging(self, receiver: int, key: str, dtype: torch.dtype, staging: torch.Tensor,
                          segments: Dict[int, Tuple[int, List[int]]]) -> None:
         self._staging[(receiver, key, dtype)] = (staging, segments)
+        self.epoch += 1
 
     def staging_segment(self, receiver: int, key: str, dtype: torch.dtype, sender: int):
         """``(staging tensor, element offset, block numels)`` of what ``receiver`` expects from
@@ -58,6 +60,7 @@ class LocalFabric:
         """Drop what ``receiver`` registered (its plan is being prepared again)."""
         for k in [k for k in self._staging if k[0] == receiver]:
             del self._staging[k]
+        self.epoch += 1
 
     # -- execute time ----------------------------------------------------------------------
     def post(self, sender: int, receiver: int, key: str, event: torch.cuda.Event) -> None:
