@@ -85,6 +85,10 @@ class LocalLayout:
             sl = [slice(t0, t0 + n_tok)] + [slice(None)] * (x.dim() - 1)
             sl[head_axis] = slice(head_block * hb, (head_block + 1) * hb)
             parts.append(x[tuple(sl)])
+        if not parts:  # a device that owns no block
+            shape = list(x.shape)
+            shape[0], shape[head_axis] = 0, hb
+            return x.new_zeros(shape)
         return torch.cat(parts, dim=0).contiguous()
 
     def to_local_q(self, q: torch.Tensor) -> torch.Tensor:
@@ -137,6 +141,8 @@ class LocalLayout:
         for head_block, seq, blk, n_tok in self.q_blocks:
             t0 = int(off[seq]) + blk * self.block_size
             parts.append(lse[head_block * hb : (head_block + 1) * hb, t0 : t0 + n_tok])
+        if not parts:
+            return lse.new_zeros((hb, 0))
         return torch.cat(parts, dim=1).contiguous()
 
 

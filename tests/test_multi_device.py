@@ -146,3 +146,33 @@ def test_fabric_staging_registry():
     fabric.forget(3)
     with pytest.raises(RuntimeError, match="no matching receives"):
         fabric.staging_segment(3, "S0", torch.bfloat16, 1)
+
+
+def _random_multi_config(rng, head_dims=(16,)):
+    n_dev = int(rng.integers(2, 6))
+    n_nodes = 2 if n_dev % 2 == 0 and rng.random() < 0.5 else 1
+    block_size = 64
+    n_seq = int(rng.integers(1, 4))
+    seqlens = [int(rng.integers(block_size + 1, 6 * block_size)) for _ in range(n_seq)]
+    n_groups = int(rng.choice([1, 2, 4]))
+    group = int(rng.choice([1, 2, 4]))
+    n_heads = n_groups * group
+    head_block = int(rng.choice([h for h in (1, 2, 4) if (group % h == 0 if group > 1 else n_heads % h == 0)]))
+    mask = str(rng.choice(["causal", "lambda"]))
+    cfg = dict(n_nodes=n_nodes, n_devices_per_node=n_dev // n_nodes, seqlens=seqlens, block_size=block_size,
+               n_heads=n_heads, n_groups=n_groups, head_dim=int(rng.choice(head_dims)), head_block=head_block, mask=mask)
+    if mask == "lambda":
+        cfg["mask_info"] = [int(rng.integers(1, 40)), int(rng.integers(40, 200))]
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_placements_reproduce_dense_attention(seed):
+    cfg = _random_multi_config(np.random.default_rng(1000 + seed))
+    case = make_multi_case(seed=seed, **cfg)
+    out, lse, dq, dkv = run_multi_oracle(case, backward=True)
+    t_out, t_lse, t_dq, t_dkv = dense_truth(case, backward=True)
+    assert np.abs(out.numpy() - t_out).max() < 3e-2, cfg
+    assert np.abs(lse.numpy() - t_lse).max() < 1e-5, cfg
+    for got, want in ((dq.numpy(), t_dq), (dkv.numpy(), t_dkv)):
+        assert (np.abs(got - want) <= 4e-2 * np.maximum(1.0, np.abs(want)) + 1e-2 * np.abs(want).max()).all(), cfg
