@@ -354,3 +354,352 @@ def build_multi_device_plans(
         return plans
 
     return build(False), build(True), layouts
+
+
+def build_staged_multi_device_plans(
+    n_nodes: int,
+    n_devices_per_node: int,
+    raw_seqlens: Sequence[int],
+    block_size: int,
+    n_heads: int,
+    n_query_groups: int,
+    head_dim: int,
+    head_block_size: int,
+    attn_mask: torch.Tensor,
+    dtype: torch.dtype = torch.bfloat16,
+    n_stages: int = 2,
+    disable_two_phase_comm: bool = False,
+):
+    """The same placement as ``build_multi_device_plans``, but the work units are grouped into
+    pipeline stages by the stage packer (``dcp_amd.core.pipeline.generate_pipelines_n_stages``):
+    stage 0 holds what needs no transfer, the blocks of stage k+1 travel (key ``S{k+1}``) while
+    stage k is computed, and a remote block wanted by several devices of a node is received by
+    one of them and forwarded inside the node on the second-phase stream (key ``S{k+1}P2``), in
+    the instruction order of ``dcp/core/scheduler.py:894-1049``.  Every (row, stage) writes its
+    own partial; partials meet at the owner of their block through the output exchange ``O``.
+    Slots are never reused.  Returns ``(fw_plans, bw_plans, layouts)`` as the unstaged builder."""
+    from types import SimpleNamespace
+
+    from dcp_amd.core.pipeline import generate_pipelines_n_stages
+
+    raw_seqlens = [int(x) for x in raw_seqlens]
+    n_dev = n_nodes * n_devices_per_node
+    group = n_heads // n_query_groups
+    assert n_heads % n_query_groups == 0 and n_heads % head_block_size == 0
+    if group > 1:
+        assert head_block_size <= group and group % head_block_size == 0
+    hb = head_block_size
+    hkv = 1 if group > 1 else head_block_size
+    n_hb_q, n_hb_kv = n_heads // hb, n_query_groups // hkv
+    q_per_kv = n_hb_q // n_hb_kv
+    mask_np = attn_mask.cpu().numpy()
+    assert mask_np.shape[0] == sum(raw_seqlens)
+    seq_off = np.concatenate(([0], np.cumsum(raw_seqlens)))
+    n_blocks_of = [(L + block_size - 1) // block_size for L in raw_seqlens]
+    wire_dtype = torch_dtype_to_int(dtype)
+    elem = 4 if dtype == torch.float32 else 2
+
+    def n_tok(s, b):
+        return min(block_size, raw_seqlens[s] - b * block_size)
+
+    def owner(s, b):
+        return divmod((s + b) % n_dev, n_devices_per_node)
+
+    def rank_of(device):
+        return device[0] * n_devices_per_node + device[1]
+
+    devices = [divmod(r, n_devices_per_node) for r in range(n_dev)]
+    q_tok_shape, kv_tok_shape = (hb, head_dim), (2, hkv, head_dim)
+    q_numel, kv_numel = block_size * hb * head_dim, block_size * 2 * hkv * head_dim
+
+    # ---- LOCAL layouts (as the unstaged builder) ------------------------------------------
+    layouts, local_index = [], []
+    for r in range(n_dev):
+        lay = LocalLayout(raw_seqlens, block_size, n_heads, n_query_groups, head_dim, hb, hkv)
+        index = {}
+        for kind, n_hb, blocks in (("q", n_hb_q, lay.q_blocks), ("kv", n_hb_kv, lay.kv_blocks)):
+            for g in range(n_hb):
+                for s in range(len(raw_seqlens)):
+                    for b in range(n_blocks_of[s]):
+                        if rank_of(owner(s, b)) == r:
+                            index[(kind, g, s, b)] = len(blocks)
+                            blocks.append((g, s, b, n_tok(s, b)))
+        cu = [0]
+        for _, _, _, n in lay.q_blocks:
+            cu.append(cu[-1] + n)
+        lay.local_cu_seqlens = cu
+        layouts.append(lay)
+        local_index.append(index)
+
+    _LOCAL = {"Q": BufferType.LOCAL_Q, "KV": BufferType.LOCAL_KV, "OUT": BufferType.LOCAL_OUT,
+              "LSE": BufferType.LOCAL_LSE, "dOUT": BufferType.LOCAL_dOUT}
+    _SLOT = {"Q": BufferType.BUFFER_Q, "KV": BufferType.BUFFER_KV, "OUT": BufferType.BUFFER_OUT,
+             "LSE": BufferType.BUFFER_LSE, "dOUT": BufferType.BUFFER_dOUT}
+
+    def build(is_bw):
+        # ---- the planning problem: data blocks, work units, where they are ----------------
+        inputs: List[Tuple[str, int, int, int]] = []  # (type, head block, sequence, block)
+        input_id: Dict[Tuple[str, int, int, int], int] = {}
+
+        def add_input(kind, g, s, b):
+            input_id[(kind, g, s, b)] = len(inputs)
+            inputs.append((kind, g, s, b))
+
+        for s in range(len(raw_seqlens)):
+            for b in range(n_blocks_of[s]):
+                for g in range(n_hb_q):
+                    add_input("Q", g, s, b)
+                    if is_bw:
+                        for kind in ("OUT", "LSE", "dOUT"):
+                            add_input(kind, g, s, b)
+                for g in range(n_hb_kv):
+                    add_input("KV", g, s, b)
+        size_of = {"Q": q_numel * elem, "OUT": q_numel * elem, "dOUT": q_numel * elem, "KV": kv_numel * elem,
+                   "LSE": block_size * hb * 4}
+        input_sizes = [float(size_of[kind]) for kind, _, _, _ in inputs]
+        input_device = {i: owner(s, b) for i, (_, _, s, b) in enumerate(inputs)}
+        units: List[Tuple[int, int, int, int]] = []  # (q head block, sequence, q block, kv block)
+        unit_inputs, unit_device, unit_cost = [], {}, []
+        for s, L in enumerate(raw_seqlens):
+            seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
+            for i in range(n_blocks_of[s]):
+                for j in _block_overlaps(seq_mask, i * block_size, n_tok(s, i), block_size, n_blocks_of[s], L):
+                    for g in range(n_hb_q):
+                        w = len(units)
+                        units.append((g, s, i, j))
+                        ins = [input_id[("Q", g, s, i)], input_id[("KV", g // q_per_kv, s, j)]]
+                        if is_bw:
+                            ins += [input_id[(kind, g, s, i)] for kind in ("OUT", "LSE", "dOUT")]
+                        unit_inputs.append(ins)
+                        unit_device[w] = owner(s, i) if (i + j) % 2 == 0 else owner(s, j)
+                        unit_cost.append(float(n_tok(s, i) * n_tok(s, j)))
+        meta = {i: SimpleNamespace(type=kind) for i, (kind, _, _, _) in enumerate(inputs)}
+        work_per_stage, first_phase, second_phase = generate_pipelines_n_stages(
+            n_stages, set(devices), unit_cost, unit_inputs, meta, input_sizes, unit_device, input_device, is_bw,
+            disable_two_phase_comm=disable_two_phase_comm)
+
+        # ---- per device: where each block it holds sits ----------------------------------------
+        slots = [{t: _Slots() for t in ("Q", "KV", "O", "out", "dq", "dkv")} for _ in range(n_dev)]
+        held: List[Dict[int, BufferBlock]] = [{} for _ in range(n_dev)]  # input id -> the block to read it from
+        o_slot: List[Dict[Key, int]] = [{} for _ in range(n_dev)]         # OUT / LSE / dOUT of a q block share a slot index
+
+        def block_of(i, buffer_type, index):
+            _, _, s, b = inputs[i]
+            return BufferBlock(buffer_type, index, n_tok(s, b))
+
+        def take_slot(r, i):
+            kind, g, s, b = inputs[i]
+            if kind in ("OUT", "LSE", "dOUT"):
+                if (g, s, b) not in o_slot[r]:
+                    o_slot[r][(g, s, b)] = slots[r]["O"].take()
+                return o_slot[r][(g, s, b)]
+            return slots[r][kind].take()
+
+        def local_block(r, i):
+            kind, g, s, b = inputs[i]
+            return block_of(i, _LOCAL[kind], local_index[r][("kv" if kind == "KV" else "q", g, s, b)])
+
+        instrs: List[list] = [[] for _ in range(n_dev)]
+        used = [set() for _ in range(n_dev)]  # inputs some work unit on the device reads
+        for stage in work_per_stage:
+            for d, ws in stage.items():
+                for w in ws:
+                    used[rank_of(d)].update(unit_inputs[w])
+        for r in range(n_dev):
+            pairs = []
+            for i in sorted(used[r]):
+                if rank_of(input_device[i]) == r:
+                    dst = block_of(i, _SLOT[inputs[i][0]], take_slot(r, i))
+                    pairs.append((local_block(r, i), dst))
+                    held[r][i] = dst
+            if pairs:
+                instrs[r].append(MemcpyInstr(pairs))
+
+        def source_block(r, i):
+            """What a device sends for input i: its own unpadded block, or the slot it received it in."""
+            return local_block(r, i) if rank_of(input_device[i]) == r else held[r][i]
+
+        def exchange_ops(transfers):
+            """transfers: (src rank, dst rank, input id) in one global order -> ops per rank."""
+            ops = [[] for _ in range(n_dev)]
+            arrivals = []
+            for src, dst, i in transfers:
+                ops[src].append(CommOp(CommType.SEND, devices[dst], source_block(src, i)))
+                slot = block_of(i, _SLOT[inputs[i][0]], take_slot(dst, i))
+                ops[dst].append(CommOp(CommType.RECV, devices[src], slot))
+                arrivals.append((dst, i, slot))
+            return ops, arrivals
+
+        partial_out = [defaultdict(list) for _ in range(n_dev)]  # q block key -> partial slots on this device
+        partial_dq = [defaultdict(list) for _ in range(n_dev)]
+        replicas = [defaultdict(list) for _ in range(n_dev)]     # kv block key -> private dKV slots
+
+        def compute(r, stage_id):
+            ws = sorted(work_per_stage[stage_id].get(devices[r], ()))
+            if not ws:
+                return
+            rows = defaultdict(list)
+            for w in ws:
+                g, s, i, j = units[w]
+                rows[(g, s, i)].append(j)
+            rows = sorted(((k, sorted(ids)) for k, ids in rows.items()), key=lambda kv: (kv[0][1], kv[0][0], kv[0][2]))
+            planes = []
+            for (g, s, i), ids in rows:
+                seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
+                planes.append(_row_ranges(seq_mask, i * block_size, n_tok(s, i), block_size, ids, [n_tok(s, j) for j in ids]))
+            m = torch.from_numpy(np.concatenate(planes, axis=2))
+            m = m[0] if m.shape[0] == 1 else m
+            seq_q = [block_size] * len(rows)
+            seq_kv = [block_size * len(ids) for _, ids in rows]
+            q_tab = [[held[r][input_id[("Q", *k)]]] for k, _ in rows]
+            kv_tab = [[held[r][input_id[("KV", k[0] // q_per_kv, k[1], j)]] for j in ids] for k, ids in rows]
+
+            def row_block(buffer_type, slot, k):
+                return BufferBlock(buffer_type, slot, n_tok(k[1], k[2]))
+
+            if not is_bw:
+                out_tab, lse_tab = [], []
+                for k, _ in rows:
+                    slot = slots[r]["out"].take()
+                    partial_out[r][k].append(slot)
+                    out_tab.append([row_block(BufferType.BUFFER_OUT, slot, k)])
+                    lse_tab.append([row_block(BufferType.BUFFER_LSE, slot, k)])
+                instrs[r].append(AttnInstr(stage_id, seq_q, seq_kv, block_size, max(seq_kv), m, q_tab, kv_tab, out_tab, lse_tab))
+                return
+            o_tab = [[row_block(BufferType.BUFFER_OUT, o_slot[r][k], k)] for k, _ in rows]
+            dq_tab, dkv_tab = [], []
+            for k, ids in rows:
+                slot = slots[r]["dq"].take()
+                partial_dq[r][k].append(slot)
+                dq_tab.append([row_block(BufferType.BUFFER_dQ, slot, k)])
+                row = []
+                for j in ids:
+                    kk = (k[0] // q_per_kv, k[1], j)
+                    slot = slots[r]["dkv"].take()
+                    replicas[r][kk].append(slot)
+                    row.append(row_block(BufferType.BUFFER_dKV, slot, kk))
+                dkv_tab.append(row)
+            instrs[r].append(AttnBackwardInstr(stage_id, seq_q, seq_kv, block_size, max(seq_kv), m, q_tab, kv_tab, o_tab, dq_tab, dkv_tab))
+
+        # ---- stages: the transfers of stage k+1 are launched before stage k is computed ---------
+        for k in range(n_stages + 1):
+            nxt = k + 1
+            waits = [[] for _ in range(n_dev)]
+            if nxt <= n_stages:
+                first = [(rank_of(src), rank_of(dst), i) for dst in sorted(first_phase[nxt]) for i, src in first_phase[nxt][dst]]
+                second = [(rank_of(src), rank_of(dst), i) for dst in sorted(second_phase[nxt]) for i, src in second_phase[nxt][dst]]
+                ops1, arrived1 = exchange_ops(first)
+                relays = {src for src, _, _ in second}
+                for r in range(n_dev):
+                    if ops1[r]:
+                        instrs[r].append(CommLaunchInstr(f"S{nxt}", ops1[r]))
+                # a relay forwards what it has just received: its receive must be booked first
+                for dst, i, slot in arrived1:
+                    held[dst][i] = slot
+                ops2, arrived2 = exchange_ops(second)
+                for r in range(n_dev):
+                    if ops2[r]:
+                        if ops1[r] and r in relays:
+                            instrs[r].append(CommWaitInstr(f"S{nxt}", stream="second_phase"))
+                        elif ops1[r]:
+                            waits[r].append(f"S{nxt}")
+                        instrs[r].append(CommLaunchInstr(f"S{nxt}P2", ops2[r], stream="second_phase"))
+                        waits[r].append(f"S{nxt}P2")
+                    elif ops1[r]:
+                        waits[r].append(f"S{nxt}")
+                for dst, i, slot in arrived2:
+                    held[dst][i] = slot
+            # stage k reads only blocks booked before this iteration's transfers: compute it now
+            # (held already names the stage k+1 arrivals, but no work unit of stage k uses them)
+            for r in range(n_dev):
+                compute(r, k)
+                for key in waits[r]:
+                    instrs[r].append(CommWaitInstr(key))
+
+        # ---- results travel to the owners of their blocks -------------------------------------
+        _RES = {"out": BufferType.BUFFER_OUT, "lse": BufferType.BUFFER_LSE, "dq": BufferType.BUFFER_dQ, "dkv": BufferType.BUFFER_dKV}
+
+        def res_block(what, slot, key):
+            return BufferBlock(_RES[what], slot, n_tok(key[1], key[2]))
+
+        if is_bw:  # one partial per block and device: sum the device's own first
+            for r in range(n_dev):
+                pre = [SumOp([res_block("dq", s_, k) for s_ in sl], res_block("dq", sl[0], k)) for k, sl in partial_dq[r].items() if len(sl) > 1]
+                pre += [SumOp([res_block("dkv", s_, k) for s_ in sl], res_block("dkv", sl[0], k)) for k, sl in replicas[r].items() if len(sl) > 1]
+                if pre:
+                    instrs[r].append(SumInstr(pre, output_is_unpadded=0))
+        o_ops = [[] for _ in range(n_dev)]
+        gathered = [defaultdict(list) for _ in range(n_dev)]  # owner: (what, key) -> slots to merge / sum
+        by_key = lambda kv: (kv[0][1], kv[0][0], kv[0][2])
+        for r in range(n_dev):
+            tables = [("dq", partial_dq[r]), ("dkv", replicas[r])] if is_bw else [("out", partial_out[r])]
+            for what, table in tables:
+                for key, sl in sorted(table.items(), key=by_key):
+                    dst = rank_of(owner(key[1], key[2]))
+                    for slot in (sl[:1] if is_bw else sl):
+                        if dst == r:
+                            gathered[r][(what, key)].append(slot)
+                            continue
+                        there = slots[dst][what].take()
+                        gathered[dst][(what, key)].append(there)
+                        for part in (("out", "lse") if what == "out" else (what,)):
+                            o_ops[r].append(CommOp(CommType.SEND, devices[dst], res_block(part, slot, key)))
+                            o_ops[dst].append(CommOp(CommType.RECV, devices[r], res_block(part, there, key)))
+        plans = []
+        for r in range(n_dev):
+            lay = layouts[r]
+            if o_ops[r]:
+                instrs[r] += [CommLaunchInstr("O", o_ops[r]), CommWaitInstr("O")]
+            finals = []
+            for (kind, g, s, b), li in local_index[r].items():
+                key = (g, s, b)
+                if kind == "q" and not is_bw and gathered[r][("out", key)]:
+                    finals.append(ReductionOp([(res_block("out", s_, key), res_block("lse", s_, key)) for s_ in gathered[r][("out", key)]],
+                                              (BufferBlock(BufferType.LOCAL_OUT, li, n_tok(s, b)), BufferBlock(BufferType.LOCAL_LSE, li, n_tok(s, b)))))
+            if finals:
+                instrs[r].append(AttnReductionInstr(finals, output_is_unpadded=1))
+            if is_bw:
+                for kind, what, local in (("q", "dq", BufferType.LOCAL_dQ), ("kv", "dkv", BufferType.LOCAL_dKV)):
+                    sums = [SumOp([res_block(what, s_, (g, s, b)) for s_ in gathered[r][(what, (g, s, b))]],
+                                  BufferBlock(local, li, n_tok(s, b)))
+                            for (k2, g, s, b), li in local_index[r].items() if k2 == kind and gathered[r][(what, (g, s, b))]]
+                    if sums:
+                        instrs[r].append(SumInstr(sums, output_is_unpadded=1))
+            total_q, total_kv = lay.local_cu_seqlens[-1], sum(n for _, _, _, n in lay.kv_blocks)
+
+            def local_info(n_blocks, total, tok_shape, numel):
+                return BufferInfo(n_blocks, block_size, numel, wire_dtype, (total, *tok_shape), tok_shape)
+
+            def slot_info(n, tok_shape, numel):
+                n = max(n, 1)
+                return BufferInfo(n, block_size, numel, wire_dtype, (n, block_size, *tok_shape), tok_shape)
+
+            def lse_slot_info(n):
+                n = max(n, 1)
+                return BufferInfo(n, block_size, block_size * hb, DType.FLOAT32, (hb, n, block_size), (1,))
+
+            n_o = slots[r]["O"].n if is_bw else slots[r]["out"].n
+            info = {
+                BufferType.LOCAL_Q: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
+                BufferType.LOCAL_KV: local_info(len(lay.kv_blocks), total_kv, kv_tok_shape, kv_numel),
+                BufferType.LOCAL_OUT: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
+                BufferType.LOCAL_LSE: BufferInfo(len(lay.q_blocks), block_size, block_size * hb, DType.FLOAT32, (hb, total_q), (1,)),
+                BufferType.BUFFER_Q: slot_info(slots[r]["Q"].n, q_tok_shape, q_numel),
+                BufferType.BUFFER_KV: slot_info(slots[r]["KV"].n, kv_tok_shape, kv_numel),
+                BufferType.BUFFER_OUT: slot_info(n_o, q_tok_shape, q_numel),
+                BufferType.BUFFER_LSE: lse_slot_info(n_o),
+            }
+            if is_bw:
+                info.update({
+                    BufferType.LOCAL_dOUT: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
+                    BufferType.LOCAL_dQ: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
+                    BufferType.LOCAL_dKV: local_info(len(lay.kv_blocks), total_kv, kv_tok_shape, kv_numel),
+                    BufferType.BUFFER_dOUT: slot_info(n_o, q_tok_shape, q_numel),
+                    BufferType.BUFFER_dQ: slot_info(slots[r]["dq"].n, q_tok_shape, q_numel),
+                    BufferType.BUFFER_dKV: slot_info(slots[r]["dkv"].n, kv_tok_shape, kv_numel),
+                })
+            node, dev = devices[r]
+            plans.append(ExecutionPlan(instrs[r], n_nodes, n_devices_per_node, node, dev, n_stages + 1, lay.local_cu_seqlens, info))
+        return plans
+
+    return build(False), build(True), layouts

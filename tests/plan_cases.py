@@ -94,12 +94,20 @@ def run_plan_oracle(case, backward=False):
 
 
 def make_multi_case(n_nodes, n_devices_per_node, seqlens, block_size, n_heads, n_groups, head_dim, head_block,
-                    mask="causal", mask_info=None, dtype="bf16", seed=0, mask_kwargs=None):
-    from dcp_amd.runtime.flash_attention.multi_device import build_multi_device_plans
+                    mask="causal", mask_info=None, dtype="bf16", seed=0, mask_kwargs=None, n_stages=None,
+                    disable_two_phase_comm=False):
+    """``n_stages`` = None: one input exchange (build_multi_device_plans); a number: the stage
+    packer groups the work units into that many stages (build_staged_multi_device_plans)."""
+    from dcp_amd.runtime.flash_attention.multi_device import build_multi_device_plans, build_staged_multi_device_plans
 
     mask_t = MASK_FNS[mask](list(seqlens), list(seqlens), torch.int32, mask_info, **(mask_kwargs or {}))
-    fw, bw, layouts = build_multi_device_plans(n_nodes, n_devices_per_node, seqlens, block_size, n_heads, n_groups,
-                                               head_dim, head_block, mask_t, dtype=TORCH_DTYPE[dtype])
+    if n_stages is None:
+        fw, bw, layouts = build_multi_device_plans(n_nodes, n_devices_per_node, seqlens, block_size, n_heads, n_groups,
+                                                   head_dim, head_block, mask_t, dtype=TORCH_DTYPE[dtype])
+    else:
+        fw, bw, layouts = build_staged_multi_device_plans(
+            n_nodes, n_devices_per_node, seqlens, block_size, n_heads, n_groups, head_dim, head_block, mask_t,
+            dtype=TORCH_DTYPE[dtype], n_stages=n_stages, disable_two_phase_comm=disable_two_phase_comm)
     g = torch.Generator().manual_seed(seed)
     T = sum(seqlens)
     q = torch.randn(T, n_heads, head_dim, generator=g).to(TORCH_DTYPE[dtype])

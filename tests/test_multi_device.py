@@ -176,3 +176,69 @@ def test_random_placements_reproduce_dense_attention(seed):
     assert np.abs(lse.numpy() - t_lse).max() < 1e-5, cfg
     for got, want in ((dq.numpy(), t_dq), (dkv.numpy(), t_dkv)):
         assert (np.abs(got - want) <= 4e-2 * np.maximum(1.0, np.abs(want)) + 1e-2 * np.abs(want).max()).all(), cfg
+
+
+# ---------------------------------------------------------------------------
+# stages laid out by the stage packer
+# ---------------------------------------------------------------------------
+
+STAGED = {
+    "two_nodes_of_three_lambda": dict(n_nodes=2, n_devices_per_node=3, seqlens=[640, 500], block_size=64, n_heads=2,
+                                      n_groups=2, head_dim=16, head_block=1, mask="lambda", mask_info=[16, 96], n_stages=2),
+    "two_nodes_of_two_gqa": dict(n_nodes=2, n_devices_per_node=2, seqlens=[900, 300], block_size=64, n_heads=4,
+                                 n_groups=1, head_dim=16, head_block=2, n_stages=2),
+    "two_nodes_of_four_four_stages": dict(n_nodes=2, n_devices_per_node=4, seqlens=[1024], block_size=64, n_heads=2,
+                                          n_groups=2, head_dim=16, head_block=2, n_stages=4),
+    "one_node_three_stages": dict(n_nodes=1, n_devices_per_node=3, seqlens=[300, 150, 260], block_size=64, n_heads=8,
+                                  n_groups=2, head_dim=16, head_block=2, n_stages=3),
+    "single_phase_only": dict(n_nodes=2, n_devices_per_node=3, seqlens=[640, 500], block_size=64, n_heads=2,
+                              n_groups=2, head_dim=16, head_block=1, n_stages=2, disable_two_phase_comm=True),
+}
+
+
+def _comm_keys(plans):
+    keys = {}
+    for p in plans:
+        for i in p.instructions:
+            if isinstance(i, (CommLaunchInstr, CommWaitInstr)):
+                k = (type(i).__name__, i.key, i.stream)
+                keys[k] = keys.get(k, 0) + 1
+    return keys
+
+
+@pytest.mark.parametrize("name", sorted(STAGED))
+def test_staged_plans_reproduce_dense_attention(name):
+    case = make_multi_case(**STAGED[name])
+    out, lse, dq, dkv = run_multi_oracle(case, backward=True)
+    t_out, t_lse, t_dq, t_dkv = dense_truth(case, backward=True)
+    assert np.abs(out.numpy() - t_out).max() < 3e-2
+    assert np.abs(lse.numpy() - t_lse).max() < 1e-5
+    for got, want in ((dq.numpy(), t_dq), (dkv.numpy(), t_dkv)):
+        assert (np.abs(got - want) <= 4e-2 * np.maximum(1.0, np.abs(want)) + 1e-2 * np.abs(want).max()).all()
+
+
+def test_staged_plans_have_the_references_instruction_structure():
+    """Stage k+1's transfers are launched before stage k's attention and waited for after it; a
+    relay waits for the first phase on the second-phase stream and forwards from there
+    (dcp/core/scheduler.py:894-1049)."""
+    from dcp_amd.core.instructions import AttnInstr
+
+    case = make_multi_case(**STAGED["two_nodes_of_three_lambda"])
+    keys = _comm_keys(case["fw"])
+    assert keys[("CommLaunchInstr", "S1P2", "second_phase")] > 0 and keys[("CommWaitInstr", "S1", "second_phase")] > 0
+    assert not any(k[0] == "CommLaunchInstr" and k[1].endswith("P2") and k[2] is None for k in keys)
+    for plan in case["fw"]:
+        names = [(type(i).__name__, getattr(i, "key", getattr(i, "stage_id", None))) for i in plan.instructions]
+        for stage in (1, 2):
+            launch = names.index(("CommLaunchInstr", f"S{stage}")) if ("CommLaunchInstr", f"S{stage}") in names else None
+            attn_before = names.index(("AttnInstr", stage - 1)) if ("AttnInstr", stage - 1) in names else None
+            attn_after = names.index(("AttnInstr", stage)) if ("AttnInstr", stage) in names else None
+            waits = [n for n, x in enumerate(names) if x[0] == "CommWaitInstr" and x[1] in (f"S{stage}", f"S{stage}P2")]
+            if launch is not None and attn_before is not None:
+                assert launch < attn_before
+            if attn_after is not None and waits:
+                assert max(waits) < attn_after
+        assert sum(isinstance(i, AttnInstr) for i in plan.instructions) <= 3
+    # without the second phase nothing runs on a side stream
+    single = _comm_keys(make_multi_case(**STAGED["single_phase_only"])["fw"])
+    assert all(k[2] is None for k in single)

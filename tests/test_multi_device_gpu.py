@@ -193,3 +193,33 @@ def test_random_placements_against_oracle(seed):
     for got, want in ((dq, o_dq), (dkv, o_dkv)):
         err = (got.float() - want.float()).abs()
         assert (err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * want.float().abs().max()).all()
+
+
+STAGED = {
+    "two_nodes_of_three_lambda": dict(n_nodes=2, n_devices_per_node=3, seqlens=[640, 500], block_size=64, n_heads=2,
+                                      n_groups=2, head_dim=64, head_block=1, mask="lambda", mask_info=[16, 96], n_stages=2),
+    "two_nodes_of_two_gqa": dict(n_nodes=2, n_devices_per_node=2, seqlens=[900, 300], block_size=64, n_heads=4,
+                                 n_groups=1, head_dim=128, head_block=2, n_stages=2),
+    "two_nodes_of_four_four_stages": dict(n_nodes=2, n_devices_per_node=4, seqlens=[2048], block_size=128, n_heads=4,
+                                          n_groups=4, head_dim=128, head_block=2, n_stages=4, dtype="fp16"),
+    "one_node_three_stages": dict(n_nodes=1, n_devices_per_node=3, seqlens=[300, 150, 260], block_size=64, n_heads=8,
+                                  n_groups=2, head_dim=64, head_block=2, n_stages=3),
+}
+
+
+@pytest.mark.parametrize("name", sorted(STAGED))
+def test_staged_exchange_matches_oracle_and_dense_attention(name):
+    """Plans whose stages the stage packer laid out: transfers of the next stage in flight while
+    a stage is computed, relays on the second-phase stream."""
+    case = make_multi_case(**STAGED[name])
+    print(f"staged multi-device case {name}", flush=True)
+    (out, lse, dq, dkv), _ = run_multi_executor(case, backward=True, repeats=2)
+    o_out, o_lse, o_dq, o_dkv = run_multi_oracle(case, backward=True)
+    t_out, t_lse, t_dq, t_dkv = dense_truth(case, backward=True)
+    for want in (o_out, torch.from_numpy(t_out)):
+        assert (out.float() - want.float()).abs().max() <= 2e-2
+    for want in (o_lse, torch.from_numpy(t_lse)):
+        assert (lse.float() - want.float()).abs().max() <= 1e-3
+    for got, want in ((dq, torch.from_numpy(t_dq)), (dkv, torch.from_numpy(t_dkv)), (dq, o_dq), (dkv, o_dkv)):
+        err = (got.float() - want.float()).abs()
+        assert (err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * want.float().abs().max()).all()
