@@ -1,11 +1,13 @@
-"""Plan builder for several devices with a fixed placement rule.
+"""Plan builders for several devices with a fixed placement rule.
 
-NOT the reference's planner (hypergraph partitioning and stage packing are out of this file's
-reach): a simple context-parallel placement that produces per-device forward and backward
+NOT the reference's planner (no hypergraph partitioning, no cost-model-driven placement, no slot
+reuse): a simple context-parallel placement that produces per-device forward and backward
 ``ExecutionPlan``s with the same instruction structure the reference scheduler emits for a
 device that exchanges blocks with others (``dcp/core/scheduler.py:894-1049`` input exchange,
 ``:1702-1762`` output exchange, ``:1764-1940`` final merges and sums), so that the
-communication instructions can be run and checked:
+communication instructions can be run and checked.  ``build_multi_device_plans`` exchanges all
+inputs at once; ``build_staged_multi_device_plans`` lets the stage packer group the work into
+pipeline stages.  The placement:
 
 * token block ``b`` of sequence ``s`` (its Q and its KV, every head block) lives on device
   ``(s + b) % n_devices``;
@@ -14,7 +16,8 @@ communication instructions can be run and checked:
   occur: KV (and Q) blocks travel to where they are multiplied, and partial results travel back
   -- (out, lse) partials to the q block's owner, which merges them, dQ partials to the q block's
   owner and dKV partials to the kv block's owner, which sum them;
-* one input exchange (key ``S0``) and one output exchange (key ``O``) per pass.
+* one input exchange (key ``S0``; ``S1``, ``S2``, ... when staged) and one output exchange
+  (key ``O``) per pass.
 
 Each device's LOCAL_* buffers hold its own blocks in (head block, sequence, block) order.
 """
