@@ -54,6 +54,129 @@ from dcp_amd.runtime.flash_attention.single_device import LocalLayout, _block_ov
 Key = Tuple[int, int, int]  # (head block, sequence, token block)
 
 
+class _Placement:
+    """What both builders share: the head blocking, the block grid of every sequence, who owns
+    which token block, each rank's LOCAL layout and the buffer descriptions."""
+
+    def __init__(self, n_nodes, n_devices_per_node, raw_seqlens, block_size, n_heads, n_query_groups, head_dim,
+                 head_block_size, attn_mask, dtype):
+        self.n_nodes, self.n_devices_per_node = n_nodes, n_devices_per_node
+        self.n_dev = n_nodes * n_devices_per_node
+        self.raw_seqlens = [int(x) for x in raw_seqlens]
+        self.block_size, self.head_dim = block_size, head_dim
+        group = n_heads // n_query_groups
+        assert n_heads % n_query_groups == 0 and n_heads % head_block_size == 0
+        if group > 1:
+            assert head_block_size <= group and group % head_block_size == 0
+        self.hb = head_block_size
+        self.hkv = 1 if group > 1 else head_block_size
+        self.n_hb_q, self.n_hb_kv = n_heads // self.hb, n_query_groups // self.hkv
+        self.q_per_kv = self.n_hb_q // self.n_hb_kv  # q head blocks sharing one kv head block
+        self.mask_np = attn_mask.cpu().numpy()
+        assert self.mask_np.shape[0] == sum(self.raw_seqlens)
+        self.seq_off = np.concatenate(([0], np.cumsum(self.raw_seqlens)))
+        self.n_blocks_of = [(L + block_size - 1) // block_size for L in self.raw_seqlens]
+        self.wire_dtype = torch_dtype_to_int(dtype)
+        self.elem_bytes = 4 if dtype == torch.float32 else 2
+        self.q_tok_shape, self.kv_tok_shape = (self.hb, head_dim), (2, self.hkv, head_dim)
+        self.q_numel, self.kv_numel = block_size * self.hb * head_dim, block_size * 2 * self.hkv * head_dim
+        # LOCAL order on every rank: (head block, sequence, block) over the blocks it owns
+        self.layouts: List[LocalLayout] = []
+        self.local_q: List[Dict[Key, int]] = []
+        self.local_kv: List[Dict[Key, int]] = []
+        for r in range(self.n_dev):
+            lay = LocalLayout(self.raw_seqlens, block_size, n_heads, n_query_groups, head_dim, self.hb, self.hkv)
+            iq, ikv = {}, {}
+            for index, n_hb, blocks in ((iq, self.n_hb_q, lay.q_blocks), (ikv, self.n_hb_kv, lay.kv_blocks)):
+                for g in range(n_hb):
+                    for s in range(len(self.raw_seqlens)):
+                        for b in range(self.n_blocks_of[s]):
+                            if self.owner(s, b) == r:
+                                index[(g, s, b)] = len(blocks)
+                                blocks.append((g, s, b, self.n_tok(s, b)))
+            cu = [0]
+            for _, _, _, n in lay.q_blocks:
+                cu.append(cu[-1] + n)
+            lay.local_cu_seqlens = cu
+            self.layouts.append(lay)
+            self.local_q.append(iq)
+            self.local_kv.append(ikv)
+
+    def n_tok(self, s, b):
+        return min(self.block_size, self.raw_seqlens[s] - b * self.block_size)
+
+    def owner(self, s, b) -> int:
+        """Rank that holds token block b of sequence s."""
+        return (s + b) % self.n_dev
+
+    def device(self, rank) -> Tuple[int, int]:
+        return divmod(rank, self.n_devices_per_node)
+
+    def unit_rank(self, s, i, j) -> int:
+        """Rank that computes (q block i, kv block j) of sequence s."""
+        return self.owner(s, i) if (i + j) % 2 == 0 else self.owner(s, j)
+
+    def attended_blocks(self, s, i) -> List[int]:
+        seq_mask = self.mask_np[self.seq_off[s] : self.seq_off[s + 1]]
+        return _block_overlaps(seq_mask, i * self.block_size, self.n_tok(s, i), self.block_size, self.n_blocks_of[s],
+                               self.raw_seqlens[s])
+
+    def rows_mask(self, rows):
+        """Range planes of attention rows ``[((g, s, i), kv block ids)]`` in their concatenated kv coordinates."""
+        planes = []
+        for (g, s, i), ids in rows:
+            seq_mask = self.mask_np[self.seq_off[s] : self.seq_off[s + 1]]
+            planes.append(_row_ranges(seq_mask, i * self.block_size, self.n_tok(s, i), self.block_size, ids,
+                                      [self.n_tok(s, j) for j in ids]))
+        t = torch.from_numpy(np.concatenate(planes, axis=2))
+        return t[0] if t.shape[0] == 1 else t
+
+    def block(self, buffer_type, index, key: Key) -> BufferBlock:
+        return BufferBlock(buffer_type, index, self.n_tok(key[1], key[2]))
+
+    def local_info(self, n_blocks, total, tok_shape, numel):
+        return BufferInfo(n_blocks, self.block_size, numel, self.wire_dtype, (total, *tok_shape), tok_shape)
+
+    def slot_info(self, n_blocks, tok_shape, numel):
+        n = max(n_blocks, 1)
+        return BufferInfo(n, self.block_size, numel, self.wire_dtype, (n, self.block_size, *tok_shape), tok_shape)
+
+    def lse_slot_info(self, n_blocks):
+        n = max(n_blocks, 1)
+        return BufferInfo(n, self.block_size, self.block_size * self.hb, DType.FLOAT32, (self.hb, n, self.block_size), (1,))
+
+    def buffer_info(self, r, n_q, n_kv, n_out, backward_slots=None):
+        """Buffer descriptions of rank r: ``n_q`` / ``n_kv`` / ``n_out`` padded slots; in the
+        backward ``backward_slots = (n_dq, n_dkv)`` and BUFFER_OUT / LSE / dOUT share ``n_out``."""
+        lay = self.layouts[r]
+        total_q, total_kv = lay.local_cu_seqlens[-1], sum(n for _, _, _, n in lay.kv_blocks)
+        nq, nkv = len(lay.q_blocks), len(lay.kv_blocks)
+        info = {
+            BufferType.LOCAL_Q: self.local_info(nq, total_q, self.q_tok_shape, self.q_numel),
+            BufferType.LOCAL_KV: self.local_info(nkv, total_kv, self.kv_tok_shape, self.kv_numel),
+            BufferType.LOCAL_OUT: self.local_info(nq, total_q, self.q_tok_shape, self.q_numel),
+            BufferType.LOCAL_LSE: BufferInfo(nq, self.block_size, self.block_size * self.hb, DType.FLOAT32, (self.hb, total_q), (1,)),
+            BufferType.BUFFER_Q: self.slot_info(n_q, self.q_tok_shape, self.q_numel),
+            BufferType.BUFFER_KV: self.slot_info(n_kv, self.kv_tok_shape, self.kv_numel),
+            BufferType.BUFFER_OUT: self.slot_info(n_out, self.q_tok_shape, self.q_numel),
+            BufferType.BUFFER_LSE: self.lse_slot_info(n_out),
+        }
+        if backward_slots is not None:
+            n_dq, n_dkv = backward_slots
+            info.update({
+                BufferType.LOCAL_dOUT: self.local_info(nq, total_q, self.q_tok_shape, self.q_numel),
+                BufferType.LOCAL_dQ: self.local_info(nq, total_q, self.q_tok_shape, self.q_numel),
+                BufferType.LOCAL_dKV: self.local_info(nkv, total_kv, self.kv_tok_shape, self.kv_numel),
+                BufferType.BUFFER_dOUT: self.slot_info(n_out, self.q_tok_shape, self.q_numel),
+                BufferType.BUFFER_dQ: self.slot_info(n_dq, self.q_tok_shape, self.q_numel),
+                BufferType.BUFFER_dKV: self.slot_info(n_dkv, self.kv_tok_shape, self.kv_numel),
+            })
+        return info
+
+
+_BY_SEQUENCE = lambda kv: (kv[0][1], kv[0][0], kv[0][2])  # rows in (sequence, head block, block) order
+
+
 def build_multi_device_plans(
     n_nodes: int,
     n_devices_per_node: int,
@@ -71,91 +194,24 @@ def build_multi_device_plans(
     ``build_single_device_plans``.  ``layouts[rank]`` maps between global tensors and the rank's
     LOCAL buffers; blocks a rank does not own come out of its ``from_local_*`` as zeros, so the
     global result is the sum over ranks."""
-    raw_seqlens = [int(x) for x in raw_seqlens]
-    n_dev = n_nodes * n_devices_per_node
-    group = n_heads // n_query_groups
-    assert n_heads % n_query_groups == 0 and n_heads % head_block_size == 0
-    if group > 1:
-        assert head_block_size <= group and group % head_block_size == 0
-    hb = head_block_size
-    hkv = 1 if group > 1 else head_block_size
-    n_hb_q, n_hb_kv = n_heads // hb, n_query_groups // hkv
-    q_per_kv = n_hb_q // n_hb_kv
-    mask_np = attn_mask.cpu().numpy()
-    assert mask_np.shape[0] == sum(raw_seqlens)
-    seq_off = np.concatenate(([0], np.cumsum(raw_seqlens)))
-    n_blocks_of = [(L + block_size - 1) // block_size for L in raw_seqlens]
-    wire_dtype = torch_dtype_to_int(dtype)
-
-    def n_tok(s, b):
-        return min(block_size, raw_seqlens[s] - b * block_size)
-
-    def owner(s, b):
-        return (s + b) % n_dev
-
-    def peer_of(rank):
-        return divmod(rank, n_devices_per_node)
+    pl = _Placement(n_nodes, n_devices_per_node, raw_seqlens, block_size, n_heads, n_query_groups, head_dim,
+                    head_block_size, attn_mask, dtype)
+    n_dev, q_per_kv, layouts, local_q, local_kv = pl.n_dev, pl.q_per_kv, pl.layouts, pl.local_q, pl.local_kv
+    owner, peer_of, blk = pl.owner, pl.device, pl.block
 
     # ---- where every work unit runs: rows[rank][(g, s, i)] = kv block ids ----------------
     rows: List[Dict[Key, List[int]]] = [defaultdict(list) for _ in range(n_dev)]
-    for s, L in enumerate(raw_seqlens):
-        seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
-        for i in range(n_blocks_of[s]):
-            for j in _block_overlaps(seq_mask, i * block_size, n_tok(s, i), block_size, n_blocks_of[s], L):
-                where = owner(s, i) if (i + j) % 2 == 0 else owner(s, j)
-                for g in range(n_hb_q):
-                    rows[where][(g, s, i)].append(j)
-
-    # ---- LOCAL layouts --------------------------------------------------------------------
-    layouts, local_q, local_kv = [], [], []
-    for r in range(n_dev):
-        lay = LocalLayout(raw_seqlens, block_size, n_heads, n_query_groups, head_dim, hb, hkv)
-        iq, ikv = {}, {}
-        for g in range(n_hb_q):
-            for s in range(len(raw_seqlens)):
-                for b in range(n_blocks_of[s]):
-                    if owner(s, b) == r:
-                        iq[(g, s, b)] = len(lay.q_blocks)
-                        lay.q_blocks.append((g, s, b, n_tok(s, b)))
-        for g in range(n_hb_kv):
-            for s in range(len(raw_seqlens)):
-                for b in range(n_blocks_of[s]):
-                    if owner(s, b) == r:
-                        ikv[(g, s, b)] = len(lay.kv_blocks)
-                        lay.kv_blocks.append((g, s, b, n_tok(s, b)))
-        cu = [0]
-        for _, _, _, n in lay.q_blocks:
-            cu.append(cu[-1] + n)
-        lay.local_cu_seqlens = cu
-        layouts.append(lay)
-        local_q.append(iq)
-        local_kv.append(ikv)
-
-    def blk(buffer_type, index, key: Key):
-        return BufferBlock(buffer_type, index, n_tok(key[1], key[2]))
-
-    def row_mask(r):
-        planes = []
-        for (g, s, i), ids in sorted(rows[r].items(), key=lambda kv: (kv[0][1], kv[0][0], kv[0][2])):
-            seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
-            planes.append(_row_ranges(seq_mask, i * block_size, n_tok(s, i), block_size, ids, [n_tok(s, j) for j in ids]))
-        t = torch.from_numpy(np.concatenate(planes, axis=2))
-        return t[0] if t.shape[0] == 1 else t
+    for s in range(len(pl.raw_seqlens)):
+        for i in range(pl.n_blocks_of[s]):
+            for j in pl.attended_blocks(s, i):
+                for g in range(pl.n_hb_q):
+                    rows[pl.unit_rank(s, i, j)][(g, s, i)].append(j)
 
     def ordered_rows(r):
-        return sorted(rows[r].items(), key=lambda kv: (kv[0][1], kv[0][0], kv[0][2]))
+        return sorted(rows[r].items(), key=_BY_SEQUENCE)
 
-    q_tok_shape, kv_tok_shape = (hb, head_dim), (2, hkv, head_dim)
-    q_numel, kv_numel = block_size * hb * head_dim, block_size * 2 * hkv * head_dim
-
-    def local_info(n_blocks, total, tok_shape, numel):
-        return BufferInfo(n_blocks, block_size, numel, wire_dtype, (total, *tok_shape), tok_shape)
-
-    def slot_info(n_blocks, tok_shape, numel):
-        return BufferInfo(n_blocks, block_size, numel, wire_dtype, (n_blocks, block_size, *tok_shape), tok_shape)
-
-    def lse_slot_info(n_blocks):
-        return BufferInfo(n_blocks, block_size, block_size * hb, DType.FLOAT32, (hb, n_blocks, block_size), (1,))
+    def row_mask(r):
+        return pl.rows_mask(ordered_rows(r))
 
     # A transfer list is built once, in one order, and read by both ends: entry
     # (src rank, dst rank, what, key) becomes a SEND in src's launch and a RECV in dst's.
@@ -304,16 +360,7 @@ def build_multi_device_plans(
             instrs = st["instrs"]
             if o_ops[r]:
                 instrs += [CommLaunchInstr("O", o_ops[r]), CommWaitInstr("O")]
-            total_q, total_kv = lay.local_cu_seqlens[-1], sum(n for _, _, _, n in lay.kv_blocks)
             slots = phase[r][0]
-            info = {
-                BufferType.LOCAL_Q: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                BufferType.LOCAL_KV: local_info(len(lay.kv_blocks), total_kv, kv_tok_shape, kv_numel),
-                BufferType.LOCAL_OUT: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                BufferType.LOCAL_LSE: BufferInfo(len(lay.q_blocks), block_size, block_size * hb, DType.FLOAT32, (hb, total_q), (1,)),
-                BufferType.BUFFER_Q: slot_info(max(slots["q"].n, 1), q_tok_shape, q_numel),
-                BufferType.BUFFER_KV: slot_info(max(slots["kv"].n, 1), kv_tok_shape, kv_numel),
-            }
             if not with_backward:
                 ops = []
                 for k, li in local_q[r].items():
@@ -323,9 +370,7 @@ def build_multi_device_plans(
                                                (blk(BufferType.LOCAL_OUT, li, k), blk(BufferType.LOCAL_LSE, li, k))))
                 if ops:
                     instrs.append(AttnReductionInstr(ops, output_is_unpadded=1))
-                n_out = max(st["res"]["out"].n, 1)
-                info[BufferType.BUFFER_OUT] = slot_info(n_out, q_tok_shape, q_numel)
-                info[BufferType.BUFFER_LSE] = lse_slot_info(n_out)
+                info = pl.buffer_info(r, slots["q"].n, slots["kv"].n, st["res"]["out"].n)
             else:
                 ops = []
                 for k, li in local_q[r].items():
@@ -341,17 +386,7 @@ def build_multi_device_plans(
                         ops.append(SumOp([blk(BufferType.BUFFER_dKV, s_, k) for s_ in srcs], blk(BufferType.LOCAL_dKV, li, k)))
                 if ops:
                     instrs.append(SumInstr(ops, output_is_unpadded=1))
-                n_o = max(slots["o"].n, 1)
-                info.update({
-                    BufferType.LOCAL_dOUT: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                    BufferType.LOCAL_dQ: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                    BufferType.LOCAL_dKV: local_info(len(lay.kv_blocks), total_kv, kv_tok_shape, kv_numel),
-                    BufferType.BUFFER_OUT: slot_info(n_o, q_tok_shape, q_numel),
-                    BufferType.BUFFER_LSE: lse_slot_info(n_o),
-                    BufferType.BUFFER_dOUT: slot_info(n_o, q_tok_shape, q_numel),
-                    BufferType.BUFFER_dQ: slot_info(max(st["res"]["dq"].n, 1), q_tok_shape, q_numel),
-                    BufferType.BUFFER_dKV: slot_info(max(st["res"]["dkv"].n, 1), kv_tok_shape, kv_numel),
-                })
+                info = pl.buffer_info(r, slots["q"].n, slots["kv"].n, slots["o"].n, (st["res"]["dq"].n, st["res"]["dkv"].n))
             node, dev = peer_of(r)
             plans.append(ExecutionPlan(instrs, n_nodes, n_devices_per_node, node, dev, 1, lay.local_cu_seqlens, info))
         return plans
@@ -385,54 +420,19 @@ def build_staged_multi_device_plans(
 
     from dcp_amd.core.pipeline import generate_pipelines_n_stages
 
-    raw_seqlens = [int(x) for x in raw_seqlens]
-    n_dev = n_nodes * n_devices_per_node
-    group = n_heads // n_query_groups
-    assert n_heads % n_query_groups == 0 and n_heads % head_block_size == 0
-    if group > 1:
-        assert head_block_size <= group and group % head_block_size == 0
-    hb = head_block_size
-    hkv = 1 if group > 1 else head_block_size
-    n_hb_q, n_hb_kv = n_heads // hb, n_query_groups // hkv
-    q_per_kv = n_hb_q // n_hb_kv
-    mask_np = attn_mask.cpu().numpy()
-    assert mask_np.shape[0] == sum(raw_seqlens)
-    seq_off = np.concatenate(([0], np.cumsum(raw_seqlens)))
-    n_blocks_of = [(L + block_size - 1) // block_size for L in raw_seqlens]
-    wire_dtype = torch_dtype_to_int(dtype)
-    elem = 4 if dtype == torch.float32 else 2
-
-    def n_tok(s, b):
-        return min(block_size, raw_seqlens[s] - b * block_size)
+    pl = _Placement(n_nodes, n_devices_per_node, raw_seqlens, block_size, n_heads, n_query_groups, head_dim,
+                    head_block_size, attn_mask, dtype)
+    n_dev, n_hb_q, n_hb_kv, q_per_kv, layouts, n_tok = pl.n_dev, pl.n_hb_q, pl.n_hb_kv, pl.q_per_kv, pl.layouts, pl.n_tok
+    devices = [pl.device(r) for r in range(n_dev)]
+    # blocks a rank owns: ("q" | "kv", head block, sequence, block) -> LOCAL index
+    local_index = [{**{("q", *k): v for k, v in pl.local_q[r].items()}, **{("kv", *k): v for k, v in pl.local_kv[r].items()}}
+                   for r in range(n_dev)]
 
     def owner(s, b):
-        return divmod((s + b) % n_dev, n_devices_per_node)
+        return devices[pl.owner(s, b)]
 
     def rank_of(device):
         return device[0] * n_devices_per_node + device[1]
-
-    devices = [divmod(r, n_devices_per_node) for r in range(n_dev)]
-    q_tok_shape, kv_tok_shape = (hb, head_dim), (2, hkv, head_dim)
-    q_numel, kv_numel = block_size * hb * head_dim, block_size * 2 * hkv * head_dim
-
-    # ---- LOCAL layouts (as the unstaged builder) ------------------------------------------
-    layouts, local_index = [], []
-    for r in range(n_dev):
-        lay = LocalLayout(raw_seqlens, block_size, n_heads, n_query_groups, head_dim, hb, hkv)
-        index = {}
-        for kind, n_hb, blocks in (("q", n_hb_q, lay.q_blocks), ("kv", n_hb_kv, lay.kv_blocks)):
-            for g in range(n_hb):
-                for s in range(len(raw_seqlens)):
-                    for b in range(n_blocks_of[s]):
-                        if rank_of(owner(s, b)) == r:
-                            index[(kind, g, s, b)] = len(blocks)
-                            blocks.append((g, s, b, n_tok(s, b)))
-        cu = [0]
-        for _, _, _, n in lay.q_blocks:
-            cu.append(cu[-1] + n)
-        lay.local_cu_seqlens = cu
-        layouts.append(lay)
-        local_index.append(index)
 
     _LOCAL = {"Q": BufferType.LOCAL_Q, "KV": BufferType.LOCAL_KV, "OUT": BufferType.LOCAL_OUT,
               "LSE": BufferType.LOCAL_LSE, "dOUT": BufferType.LOCAL_dOUT}
@@ -448,8 +448,8 @@ def build_staged_multi_device_plans(
             input_id[(kind, g, s, b)] = len(inputs)
             inputs.append((kind, g, s, b))
 
-        for s in range(len(raw_seqlens)):
-            for b in range(n_blocks_of[s]):
+        for s in range(len(pl.raw_seqlens)):
+            for b in range(pl.n_blocks_of[s]):
                 for g in range(n_hb_q):
                     add_input("Q", g, s, b)
                     if is_bw:
@@ -457,16 +457,15 @@ def build_staged_multi_device_plans(
                             add_input(kind, g, s, b)
                 for g in range(n_hb_kv):
                     add_input("KV", g, s, b)
-        size_of = {"Q": q_numel * elem, "OUT": q_numel * elem, "dOUT": q_numel * elem, "KV": kv_numel * elem,
-                   "LSE": block_size * hb * 4}
+        q_bytes, kv_bytes = pl.q_numel * pl.elem_bytes, pl.kv_numel * pl.elem_bytes
+        size_of = {"Q": q_bytes, "OUT": q_bytes, "dOUT": q_bytes, "KV": kv_bytes, "LSE": block_size * pl.hb * 4}
         input_sizes = [float(size_of[kind]) for kind, _, _, _ in inputs]
         input_device = {i: owner(s, b) for i, (_, _, s, b) in enumerate(inputs)}
         units: List[Tuple[int, int, int, int]] = []  # (q head block, sequence, q block, kv block)
         unit_inputs, unit_device, unit_cost = [], {}, []
-        for s, L in enumerate(raw_seqlens):
-            seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
-            for i in range(n_blocks_of[s]):
-                for j in _block_overlaps(seq_mask, i * block_size, n_tok(s, i), block_size, n_blocks_of[s], L):
+        for s in range(len(pl.raw_seqlens)):
+            for i in range(pl.n_blocks_of[s]):
+                for j in pl.attended_blocks(s, i):
                     for g in range(n_hb_q):
                         w = len(units)
                         units.append((g, s, i, j))
@@ -474,7 +473,7 @@ def build_staged_multi_device_plans(
                         if is_bw:
                             ins += [input_id[(kind, g, s, i)] for kind in ("OUT", "LSE", "dOUT")]
                         unit_inputs.append(ins)
-                        unit_device[w] = owner(s, i) if (i + j) % 2 == 0 else owner(s, j)
+                        unit_device[w] = devices[pl.unit_rank(s, i, j)]
                         unit_cost.append(float(n_tok(s, i) * n_tok(s, j)))
         meta = {i: SimpleNamespace(type=kind) for i, (kind, _, _, _) in enumerate(inputs)}
         work_per_stage, first_phase, second_phase = generate_pipelines_n_stages(
@@ -545,13 +544,8 @@ def build_staged_multi_device_plans(
             for w in ws:
                 g, s, i, j = units[w]
                 rows[(g, s, i)].append(j)
-            rows = sorted(((k, sorted(ids)) for k, ids in rows.items()), key=lambda kv: (kv[0][1], kv[0][0], kv[0][2]))
-            planes = []
-            for (g, s, i), ids in rows:
-                seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
-                planes.append(_row_ranges(seq_mask, i * block_size, n_tok(s, i), block_size, ids, [n_tok(s, j) for j in ids]))
-            m = torch.from_numpy(np.concatenate(planes, axis=2))
-            m = m[0] if m.shape[0] == 1 else m
+            rows = sorted(((k, sorted(ids)) for k, ids in rows.items()), key=_BY_SEQUENCE)
+            m = pl.rows_mask(rows)
             seq_q = [block_size] * len(rows)
             seq_kv = [block_size * len(ids) for _, ids in rows]
             q_tab = [[held[r][input_id[("Q", *k)]]] for k, _ in rows]
@@ -633,11 +627,10 @@ def build_staged_multi_device_plans(
                     instrs[r].append(SumInstr(pre, output_is_unpadded=0))
         o_ops = [[] for _ in range(n_dev)]
         gathered = [defaultdict(list) for _ in range(n_dev)]  # owner: (what, key) -> slots to merge / sum
-        by_key = lambda kv: (kv[0][1], kv[0][0], kv[0][2])
         for r in range(n_dev):
             tables = [("dq", partial_dq[r]), ("dkv", replicas[r])] if is_bw else [("out", partial_out[r])]
             for what, table in tables:
-                for key, sl in sorted(table.items(), key=by_key):
+                for key, sl in sorted(table.items(), key=_BY_SEQUENCE):
                     dst = rank_of(owner(key[1], key[2]))
                     for slot in (sl[:1] if is_bw else sl):
                         if dst == r:
@@ -668,39 +661,10 @@ def build_staged_multi_device_plans(
                             for (k2, g, s, b), li in local_index[r].items() if k2 == kind and gathered[r][(what, (g, s, b))]]
                     if sums:
                         instrs[r].append(SumInstr(sums, output_is_unpadded=1))
-            total_q, total_kv = lay.local_cu_seqlens[-1], sum(n for _, _, _, n in lay.kv_blocks)
-
-            def local_info(n_blocks, total, tok_shape, numel):
-                return BufferInfo(n_blocks, block_size, numel, wire_dtype, (total, *tok_shape), tok_shape)
-
-            def slot_info(n, tok_shape, numel):
-                n = max(n, 1)
-                return BufferInfo(n, block_size, numel, wire_dtype, (n, block_size, *tok_shape), tok_shape)
-
-            def lse_slot_info(n):
-                n = max(n, 1)
-                return BufferInfo(n, block_size, block_size * hb, DType.FLOAT32, (hb, n, block_size), (1,))
-
-            n_o = slots[r]["O"].n if is_bw else slots[r]["out"].n
-            info = {
-                BufferType.LOCAL_Q: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                BufferType.LOCAL_KV: local_info(len(lay.kv_blocks), total_kv, kv_tok_shape, kv_numel),
-                BufferType.LOCAL_OUT: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                BufferType.LOCAL_LSE: BufferInfo(len(lay.q_blocks), block_size, block_size * hb, DType.FLOAT32, (hb, total_q), (1,)),
-                BufferType.BUFFER_Q: slot_info(slots[r]["Q"].n, q_tok_shape, q_numel),
-                BufferType.BUFFER_KV: slot_info(slots[r]["KV"].n, kv_tok_shape, kv_numel),
-                BufferType.BUFFER_OUT: slot_info(n_o, q_tok_shape, q_numel),
-                BufferType.BUFFER_LSE: lse_slot_info(n_o),
-            }
             if is_bw:
-                info.update({
-                    BufferType.LOCAL_dOUT: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                    BufferType.LOCAL_dQ: local_info(len(lay.q_blocks), total_q, q_tok_shape, q_numel),
-                    BufferType.LOCAL_dKV: local_info(len(lay.kv_blocks), total_kv, kv_tok_shape, kv_numel),
-                    BufferType.BUFFER_dOUT: slot_info(n_o, q_tok_shape, q_numel),
-                    BufferType.BUFFER_dQ: slot_info(slots[r]["dq"].n, q_tok_shape, q_numel),
-                    BufferType.BUFFER_dKV: slot_info(slots[r]["dkv"].n, kv_tok_shape, kv_numel),
-                })
+                info = pl.buffer_info(r, slots[r]["Q"].n, slots[r]["KV"].n, slots[r]["O"].n, (slots[r]["dq"].n, slots[r]["dkv"].n))
+            else:
+                info = pl.buffer_info(r, slots[r]["Q"].n, slots[r]["KV"].n, slots[r]["out"].n)
             node, dev = devices[r]
             plans.append(ExecutionPlan(instrs[r], n_nodes, n_devices_per_node, node, dev, n_stages + 1, lay.local_cu_seqlens, info))
         return plans
