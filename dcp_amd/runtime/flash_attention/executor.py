@@ -690,7 +690,7 @@ class _CopyTables:
         for col, v in zip(self.lse, (*src, *dst, n_tokens)):
             col.append(v)
 
-    def freeze(self, exec: AttentionExecutor):
+    def freeze(self):
         data = {key: tuple(_dev(c, k) for c, k in zip(cols, _DATA_KINDS)) for key, cols in self.data.items()}
         lse = None
         if self.lse[0]:
@@ -764,7 +764,7 @@ def _prepare_comm_launch(exec: AttentionExecutor, instr: CommLaunchInstr):
         "epoch": None,
         "send_peers": sorted({peer for peer, _, _, _ in sends}),
         "recv_peers": sorted({peer for per_peer in recvs.values() for peer in per_peer}),
-        "unpack": unpack.freeze(exec),
+        "unpack": unpack.freeze(),
         "staging": staging_buffers,
     }
 
@@ -791,7 +791,7 @@ def _resolve_sends(exec: AttentionExecutor, instr: CommLaunchInstr, cache: dict)
         expected = len(exec.fabric.staging_segment(peer, instr.key, dtype, exec.rank)[2])
         if n != expected:
             raise RuntimeError(f"key {instr.key!r}: rank {exec.rank} sends {n} blocks to rank {peer}, which expects {expected}")
-    cache["pack"] = pack.freeze(exec)
+    cache["pack"] = pack.freeze()
 
 
 def _handle_comm_launch(exec: AttentionExecutor, instr: CommLaunchInstr):
