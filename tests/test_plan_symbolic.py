@@ -1,0 +1,78 @@
+"""Plans checked for structure alone by a symbolic run (tests/symbolic.py), the way the
+reference checks its compiler's output with a DummyExecutor (tests/core/test_compiler.py:137-765):
+single-device plans (one or several partials per row, folded or merged at the end) and plans for
+several devices, unstaged and staged by the stage packer."""
+
+import pytest
+import torch
+
+from dcp_amd.core.instructions import BufferBlock, CommLaunchInstr, CommOp
+from tests.plan_cases import make_case, make_multi_case
+from tests.symbolic import run_symbolic
+
+SINGLE = {
+    "causal_one_partial": dict(seqlens=[200, 330], block_size=64, n_heads=4, n_groups=4, head_dim=16, head_block=2),
+    "gqa_three_partials": dict(seqlens=[500, 130], block_size=64, n_heads=8, n_groups=2, head_dim=16, head_block=2,
+                               n_kv_groups=3),
+    "lambda_folded": dict(seqlens=[700], block_size=64, n_heads=2, n_groups=2, head_dim=16, head_block=1, mask="lambda",
+                          mask_info=[16, 96], n_kv_groups=2, kv_split="contiguous", fold=True),
+}
+MULTI = {
+    "unstaged_four_devices": dict(n_nodes=2, n_devices_per_node=2, seqlens=[300, 150, 260], block_size=64, n_heads=8,
+                                  n_groups=2, head_dim=16, head_block=2),
+    "staged_two_phase": dict(n_nodes=2, n_devices_per_node=3, seqlens=[640, 500], block_size=64, n_heads=2, n_groups=2,
+                             head_dim=16, head_block=1, mask="lambda", mask_info=[16, 96], n_stages=2),
+    "staged_four_stages": dict(n_nodes=2, n_devices_per_node=4, seqlens=[1024], block_size=64, n_heads=2, n_groups=2,
+                               head_dim=16, head_block=2, n_stages=4),
+}
+
+
+def _q_per_kv(cfg):
+    group = cfg["n_heads"] // cfg["n_groups"]
+    hkv = 1 if group > 1 else cfg["head_block"]
+    return (cfg["n_heads"] // cfg["head_block"]) // (cfg["n_groups"] // hkv)
+
+
+@pytest.mark.parametrize("name", sorted(SINGLE))
+def test_single_device_plans(name):
+    cfg = SINGLE[name]
+    case = make_case(**cfg)
+    for plan, backward in ((case["fw"], False), (case["bw"], True)):
+        run_symbolic([plan], [case["layout"]], 1, backward, case["mask"], _q_per_kv(cfg))
+
+
+@pytest.mark.parametrize("name", sorted(MULTI))
+def test_multi_device_plans(name):
+    cfg = MULTI[name]
+    case = make_multi_case(**cfg)
+    for plans, backward in ((case["fw"], False), (case["bw"], True)):
+        run_symbolic(plans, case["layouts"], case["n_devices_per_node"], backward, case["mask"], _q_per_kv(cfg))
+
+
+def test_the_checker_notices_a_wrong_plan():
+    """A kv block swapped in an attention row, a receive into the wrong kind of slot and a dropped
+    work unit must each fail."""
+    cfg = MULTI["unstaged_four_devices"]
+    args = lambda case: (case["layouts"], case["n_devices_per_node"], False, case["mask"], _q_per_kv(cfg))
+    case = make_multi_case(**cfg)
+    attn = next(i for i in case["fw"][0].instructions if type(i).__name__ == "AttnInstr")
+    row = next(r for r in attn.kv_block_table if len(r) >= 2)
+    row[0], row[1] = row[1], row[0]
+    with pytest.raises(AssertionError, match="sequence order"):
+        run_symbolic(case["fw"], *args(case))
+
+    case = make_multi_case(**cfg)
+    launch = next(i for i in case["fw"][1].instructions if isinstance(i, CommLaunchInstr) and i.key == "S0")
+    k = next(n for n, op in enumerate(launch.comm_ops) if op.comm_type == 1 and op.buffer_block.buffer_type == "BufferKV")
+    op = launch.comm_ops[k]
+    launch.comm_ops[k] = CommOp(op.comm_type, op.peer, BufferBlock("BufferQ", 0, op.buffer_block.n_tokens))
+    with pytest.raises(AssertionError):
+        run_symbolic(case["fw"], *args(case))
+
+    case = make_multi_case(**cfg)
+    attn = next(i for i in case["fw"][2].instructions if type(i).__name__ == "AttnInstr")
+    b = next(n for n, r in enumerate(attn.kv_block_table) if len(r) >= 2)
+    attn.kv_block_table[b].pop()
+    attn.seqlens_kv[b] -= 64
+    with pytest.raises(AssertionError):
+        run_symbolic(case["fw"], *args(case))
