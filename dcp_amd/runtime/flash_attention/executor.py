@@ -32,7 +32,7 @@ import math
 import numpy as np
 import torch
 
-from dcp_amd.core.executor import DCPExecutor
+from dcp_amd.core.executor import DCPExecutor, HandlerTable
 from dcp_amd.core.instructions import *  # noqa: F401,F403
 from dcp_amd.core.instructions import (
     AttnBackwardInstr,
@@ -115,7 +115,7 @@ class AttentionExecutor(DCPExecutor):
         self.head_dim = head_dim
         self.main_stream = torch.cuda.Stream()
         self.streams: Dict[str, torch.cuda.Stream] = {}
-        self._prep_handlers = {}
+        self._prep_handlers = HandlerTable("Prep handler")
         self._args_cache = {}
         self.register_synchronization_handler(torch.cuda.synchronize)
         self.fw_exec_plan = fw_exec_plan
@@ -154,14 +154,7 @@ class AttentionExecutor(DCPExecutor):
 
     # -- prepare / execute -------------------------------------------------------
     def register_prep_handler(self, instruction_type, handler):
-        if not (isinstance(instruction_type, type) and issubclass(instruction_type, BlockInstrBase)):
-            raise TypeError(
-                "Instruction type must be a subclass of BlockInstrBase, got "
-                f"{getattr(instruction_type, '__name__', instruction_type)}"
-            )
-        if instruction_type in self._prep_handlers:
-            raise ValueError(f"Prep handler for {instruction_type.__name__} already registered.")
-        self._prep_handlers[instruction_type] = handler
+        self._prep_handlers.register(instruction_type, handler)
 
     def prepare(self, forward=True):
         """Allocate the plan's buffers and build every instruction's device
