@@ -223,3 +223,37 @@ def test_staged_exchange_matches_oracle_and_dense_attention(name):
     for got, want in ((dq, torch.from_numpy(t_dq)), (dkv, torch.from_numpy(t_dkv)), (dq, o_dq), (dkv, o_dkv)):
         err = (got.float() - want.float()).abs()
         assert (err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * want.float().abs().max()).all()
+
+
+def test_a_device_that_sends_to_itself_runs_through_plain_execute():
+    """One device, its own peer: ``AttentionExecutor.execute`` needs no turn taking."""
+    from dcp_amd.core.instructions import (BufferBlock, BufferInfo, BufferType, CommLaunchInstr, CommOp, CommType,
+                                            CommWaitInstr, DType, ExecutionPlan)
+    from dcp_amd.runtime.flash_attention.executor import get_executor
+    from dcp_amd.runtime.flash_attention.fabric import LocalFabric
+
+    bs, hb, d, n = 64, 2, 64, 3
+    tokens = [bs, 17, 40]
+    cu = [0, 64, 81, 121]
+    numel = bs * hb * d
+    info = {
+        BufferType.LOCAL_Q: BufferInfo(n, bs, numel, DType.FLOAT16, (cu[-1], hb, d), (hb, d)),
+        BufferType.LOCAL_KV: BufferInfo(n, bs, 2 * numel, DType.FLOAT16, (cu[-1], 2, hb, d), (2, hb, d)),
+        BufferType.LOCAL_OUT: BufferInfo(n, bs, numel, DType.FLOAT16, (cu[-1], hb, d), (hb, d)),
+        BufferType.LOCAL_LSE: BufferInfo(n, bs, bs * hb, DType.FLOAT32, (hb, cu[-1]), (1,)),
+        BufferType.BUFFER_Q: BufferInfo(n, bs, numel, DType.FLOAT16, (n, bs, hb, d), (hb, d)),
+    }
+    ops = []
+    for i, t in enumerate(tokens):
+        ops.append(CommOp(CommType.SEND, (0, 0), BufferBlock(BufferType.LOCAL_Q, i, t)))
+        ops.append(CommOp(CommType.RECV, (0, 0), BufferBlock(BufferType.BUFFER_Q, (i + 1) % n, t)))
+    plan = ExecutionPlan([CommLaunchInstr("S0", ops), CommWaitInstr("S0")], 1, 1, 0, 0, 1, cu, info)
+    ex = get_executor(hb, d, None, fw_exec_plan=plan, fabric=LocalFabric(1, 1))
+    ex.prepare(forward=True)
+    src = torch.randn(cu[-1], hb, d).to(torch.float16)
+    ex.buffers[BufferType.LOCAL_Q].copy_(src)
+    for _ in range(2):
+        ex.execute(plan, True)
+    torch.cuda.synchronize()
+    for i, t in enumerate(tokens):
+        assert torch.equal(ex.buffers[BufferType.BUFFER_Q][(i + 1) % n, :t].cpu(), src[cu[i] : cu[i] + t])
