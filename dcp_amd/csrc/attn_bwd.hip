@@ -5,7 +5,7 @@
 //   bwd_prep_kernel      delta[q, h] = -sum_d dO*O  (negated: it is added, as an accumulator's initial value)
 //   bwd_tile_hull_kernel per (row, 64-query tile): hull and core of the rows'
 //                        key ranges, so the dK/dV kernel can skip / unmask tiles
-//   attn_bwd_dkv_kernel  key-outer: one workgroup per (row, 64-key tile, kv
+//   attn_bwd_dkv_kernel  key-outer: one workgroup per (row, 128-key tile, kv
 //                        head) loops over the q heads of the kv head's group
 //                        and the 64-query tiles of the row and keeps dK^T and
 //                        dV^T of its keys in registers
@@ -19,8 +19,9 @@
 // 64k-token causal schedule: device-scope float atomics from eight XCDs cost
 // more than the two recomputed products.
 //
-// dK/dV kernel, per step of (64 q) x (64 kv).  Wave (qi, ki) owns the 32x32
-// sub-tile (queries 32qi.., keys 32ki..) from start to end:
+// dK/dV kernel.  Wave w owns keys 32w..32w+31 of the workgroup's 128 from start
+// to end.  A step is one (q head, 64-query tile); the wave takes its two halves
+// of 32 queries one after the other (a sub-step):
 //
 //   S  = Q K^T          A = Q rows from LDS,   B = K held in registers
 //   dP = dO V^T         A = dO rows from LDS,  B = V held in registers
@@ -34,16 +35,18 @@
 //
 // P and dS never leave the registers, so a step needs one workgroup barrier (the
 // one that publishes its tiles) and LDS holds nothing but the Q and dO tiles, two
-// stages of each: everything a step reads is requested one step ahead.  The two
-// waves that share a key half (qi = 0, 1) each hold a partial dK^T/dV^T over
-// their 32 queries; they are added once, after the loop, through LDS.  The range
-// mask enters S as the accumulator's initial value (0 or -inf).  dK/dV of a key
-// never leave the workgroup until the end, so the per-(row, kv block) private
-// dKV blocks of the plan need no atomics and are written whole (zeros where no
-// query of the row attends).
+// stages of each: everything a step reads is requested one step ahead.  With four
+// waves side by side along the keys, a Q/dO tile brought into LDS, a barrier and a
+// step's scalar control serve 64 matrix instructions per wave (with two waves
+// along the keys and two along the queries it was 32, and the two query halves
+// had to be added through LDS at the end).  The range mask enters S as the
+// accumulator's initial value (0 or -inf).  dK/dV of a key never leave the wave
+// until the end, so the per-(row, kv block) private dKV blocks of the plan need
+// no atomics and are written whole (zeros where no query of the row attends).
 #include <math.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "attn_common.h"
 
@@ -90,7 +93,7 @@ struct AttnBwdParams {
   int64_t n_dq_items;    // batch * n_heads_q * dq_tiles_per_row
   int q_tiles_per_row;   // ceil(block_size / 64): query tiles of the dK/dV kernel
   int dq_tiles_per_row;  // ceil(block_size / 128): query tiles of the dQ kernel
-  int kv_tiles_per_row;  // max_kv_blocks * block_size / 64
+  int kv_tiles_per_row;  // ceil(max_kv_blocks * block_size / 128): key tiles of the dK/dV kernel
   float scale;
   float scale_log2;
 };
@@ -174,21 +177,21 @@ __global__ __launch_bounds__(64) void bwd_tile_hull_kernel(const AttnBwdParams p
 // ---------------------------------------------------------------------------
 // dK/dV kernel
 // ---------------------------------------------------------------------------
+constexpr int kDkvBN = 128;  // keys per workgroup: four waves of 32 keys each
+
 template <int DTYPE, int D>
 __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
-  constexpr int BM = kBwdBM, BN = kBwdBN;
+  constexpr int BM = kBwdBM, BN = kDkvBN;
   constexpr int KS = D / 16;  // k-steps over the head dim
   constexpr int DT = D / 32;  // 32-dim blocks of dK^T / dV^T
   typedef KvTile<D> Tile;     // the Q and dO tiles: 64 queries x D
 
-  // two stages of everything a step reads: its Q and dO tiles and the per-query scalars.
-  // After the loop the tile area is reused (as floats) for the reduction over the two
-  // query halves.
+  // two stages of everything a step reads: its Q and dO tiles and the per-query scalars
   __shared__ __attribute__((aligned(16))) uint16_t tiles[4][Tile::SIZE];  // [2 * stage + (0: Q, 1: dO)]
   __shared__ __attribute__((aligned(16))) int rng_lds[2][4][BM];  // planes: start0, end0, start1, end1
   __shared__ __attribute__((aligned(16))) float lse_lds[2][BM];
   __shared__ __attribute__((aligned(16))) float delta_lds[2][BM];
-  __shared__ unsigned long long mask_lds[2];
+  __shared__ unsigned long long mask_lds[kBwdThreads / 64];
   // With D = 128 the accumulators (128 registers), K and V (64) and the products in flight do
   // not fit in 256 registers.  The compiler would spill to scratch memory, and a scratch
   // reload waits for every outstanding global load, i.e. for the tiles requested a step
@@ -196,15 +199,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // the other operands).
   constexpr int VL = D == 128 ? 2 : 0;
   __shared__ u32x4 v_park[VL > 0 ? kBwdThreads / 64 : 1][VL > 0 ? VL : 1][64];
-  static_assert(sizeof(tiles) >= 4 * 16 * DT * 64 * sizeof(float), "reduction buffer");
 
   const int tid = threadIdx.x;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's 32 keys of the tile
   const int lane = tid & 63;
   const int c = lane & 31;
   const int h = lane >> 5;
-  const int qi = w >> 1;  // this wave's 32 queries of a step
-  const int ki = w & 1;   // this wave's 32 keys of the tile
 
   // ---- which (row, kv head, key tile) ------------------------------------------
   // the key tiles of a row share its Q/dO tiles: keep them on one XCD
@@ -223,8 +223,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
   const int k0 = kt * BN;
   if (k0 >= seqlen_kv) return;
-  const int blk = __builtin_amdgcn_readfirstlane(k0 / p.block_size);
-  const int tok0 = k0 - blk * p.block_size;
+  // A wave whose 32 keys lie past the row's keys (seqlen_kv need not be a multiple of 128) still
+  // loads its share of every tile and meets every barrier; its arithmetic is switched off and it
+  // stores nothing.  Its K/V addresses fall back to the tile's first keys so that they stay valid.
+  const int kw = k0 + w * 32;
+  const bool has_keys = kw < seqlen_kv;
+  const int kw_safe = has_keys ? kw : k0;
+  const int blk = __builtin_amdgcn_readfirstlane(kw_safe / p.block_size);
+  const int tok0 = kw_safe - blk * p.block_size;
   const int group = p.n_heads_q / p.n_heads_kv;
   const int64_t q_row_stride = (int64_t)p.n_heads_q * D;
   const int q_slot = p.q_block_table[b];
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // ---- K, V of this wave's 32 keys as B operands (lane = key, slots = dims) ------
   u32x4 kreg[KS], vreg[KS - VL];
   {
-    const int64_t off = kv_tile_off + (int64_t)(ki * 32 + c) * p.kv_token_stride + h * 8;
+    const int64_t off = kv_tile_off + (int64_t)c * p.kv_token_stride + h * 8;
     const uint16_t* kp = reinterpret_cast<const uint16_t*>(p.k) + off;
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v) + off;
 #pragma unroll
@@ -247,7 +253,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     for (int j = 0; j < VL; ++j) v_park[w][j][lane] = *reinterpret_cast<const u32x4*>(vp + (KS - VL + j) * 16);
   }
 
-  // this wave's share of dK^T and dV^T: (all dims) x (its 32 keys), summed over its query half
+  // dK^T and dV^T of this wave's keys: (all dims) x (32 keys), complete when the loop ends
   f32x16 dk_acc[DT], dv_acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -259,38 +265,33 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 
   const int32_t* hull_row = p.hull + (int64_t)b * p.q_tiles_per_row * 8;
   // loop-invariant per-lane pieces of the addresses used in the loop
-  const int row_rd = Tile::row_base(c, h) + qi * Tile::ROW32;
-  const int col_rd = Tile::col_base(lane, true) + qi * Tile::ROW32;
+  const int row_rd = Tile::row_base(c, h);
+  const int col_rd = Tile::col_base(lane, true);
   const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.block_size * q_row_stride;
   const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.block_size * q_row_stride;
   const uint32_t tiles_at = lds_address(&tiles[0][0]);
 
-  // ---- which 64-query tiles of the row see these keys (the same for every head) ----------
-  // bit qt of `act`: some row of tile qt sees some key of the tile; of `unm`: every row sees
-  // every key.  Taken once from the per-tile hulls, so the loop never waits for a table.
+  // ---- which 64-query tiles of the row see this wave's keys (the same for every head) ------
+  // bit qt of `act_w`: some row of tile qt sees some of the wave's keys; of `unm_w`: every row sees
+  // all of them.  Taken once from the per-tile hulls, so the loop never waits for a table.  The
+  // workgroup walks the tiles any of its waves needs (`act_mask`); a wave sits out the others.
+  unsigned long long act_w, unm_w;
   {
     bool a = false, u = false;
-    if (tid < 64 && tid < n_q_tiles) {
-      const int32_t* hu = hull_row + tid * 8;
-      a = (k0 < hu[1] && k0 + BN > hu[0]) || (k0 < hu[3] && k0 + BN > hu[2]);
-      u = (hu[4] <= k0 && k0 + BN <= hu[5]) || (hu[6] <= k0 && k0 + BN <= hu[7]);
+    if (has_keys && lane < n_q_tiles) {
+      const int32_t* hu = hull_row + lane * 8;
+      a = (kw < hu[1] && kw + 32 > hu[0]) || (kw < hu[3] && kw + 32 > hu[2]);
+      u = (hu[4] <= kw && kw + 32 <= hu[5]) || (hu[6] <= kw && kw + 32 <= hu[7]);
     }
-    if (w == 0) {
-      const unsigned long long am = __ballot(a), um = __ballot(u);
-      if (lane == 0) {
-        mask_lds[0] = am;
-        mask_lds[1] = um;
-      }
-    }
+    act_w = __ballot(a);
+    unm_w = __ballot(u);
+    if (lane == 0) mask_lds[w] = act_w;
   }
   __syncthreads();
-  const unsigned long long act = mask_lds[0], unm_v = mask_lds[1];
+  const unsigned long long act = mask_lds[0] | mask_lds[1] | mask_lds[2] | mask_lds[3];
   const uint32_t act_lo = __builtin_amdgcn_readfirstlane((uint32_t)act);
   const uint32_t act_hi = __builtin_amdgcn_readfirstlane((uint32_t)(act >> 32));
   const unsigned long long act_mask = ((unsigned long long)act_hi << 32) | act_lo;
-  const uint32_t unm_lo = __builtin_amdgcn_readfirstlane((uint32_t)unm_v);
-  const uint32_t unm_hi = __builtin_amdgcn_readfirstlane((uint32_t)(unm_v >> 32));
-  const unsigned long long unm = ((unsigned long long)unm_hi << 32) | unm_lo;
 
   // Everything step (head, qt) reads is requested a step ahead, straight into LDS stage st
   // and with nothing held in registers meanwhile: the Q and dO tiles, and one value per
@@ -301,7 +302,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const uint32_t goff0 = Tile::lane_offset0(q_row_stride, w, lane);
   // tile load idx of a step: the wave's group loads of the Q tile, then of the dO tile
   constexpr int NL = 2 * Tile::LPW;
-  static_assert(NL <= KS, "half of the tile loads go between the k-steps of the first phase");
+  static_assert(NL <= KS, "a sub-step carries half of the tile loads, one per two k-steps of its first phase");
   auto request_tile = [&](int idx, int head, int qt, int st) {
     const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
     const bool is_do = idx >= Tile::LPW;
@@ -341,7 +342,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   }
   while (act_mask != 0 && hg < group) {
     const int qt = __builtin_ctzll(rem);
-    const bool unmasked = (unm >> qt) & 1;
+    const bool unmasked = (unm_w >> qt) & 1;
     rem &= rem - 1;
     int hg_next = hg;
     if (rem == 0) {
@@ -352,153 +353,151 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed
-    // the next step's tiles are requested one load per k-step below: a burst here would
-    // hold the wave at its last load until the memory pipeline has taken them all
-    // They are issued unconditionally, so that the step has no branches around them: the last
-    // step requests its own tiles once more, into the stage nobody reads any more.
+    // The next step's tiles are requested one load at a time between the matrix instructions of
+    // the first phases below: a burst here would hold the wave at its last load until the memory
+    // pipeline has taken them all.  They are issued unconditionally, so that the step has no
+    // branches around them: the last step requests its own tiles once more, into the stage nobody
+    // reads any more.
     const int head_next = more ? kv_head * group + hg_next : kv_head * group + hg;
     const int qt_next = more ? __builtin_ctzll(rem) : qt;
     const uint16_t* q_lds = tiles[2 * st];
     const uint16_t* do_lds = tiles[2 * st + 1];
 
-    // ---- S = Q K^T, dP = dO V^T on this wave's 32 queries x 32 keys --------------------
-    // (A = rows of the Q / dO tile, B = K / V in registers; lane = key, element i = query
-    // 32qi + acc_row(i, h)).  The range mask enters S as the accumulator's initial value.
-    f32x16 s_acc, dp_acc;
-    const int kv = k0 + ki * 32 + c;
-    if (unmasked) {
+    // One sub-step = this wave's 32 keys against 32 of the step's 64 queries (QI = 0, 1).
+    // (A real loop, not unrolled: one copy of the body keeps the register allocation of a single
+    // sub-step; unrolled twice the compiler spills the K/V operands.)
+    auto sub_step = [&](const int QI) {
+      const int row_rd_q = row_rd + QI * Tile::ROW32, col_rd_q = col_rd + QI * Tile::ROW32;
+      // ---- S = Q K^T, dP = dO V^T on 32 queries x 32 keys ---------------------------------
+      // (A = rows of the Q / dO tile, B = K / V in registers; lane = key, element i = query
+      // 32 QI + acc_row(i, h)).  The range mask enters S as the accumulator's initial value.
+      f32x16 s_acc, dp_acc;
+      const int kv = kw + c;
+      if (unmasked) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
-    } else {
-      // the four queries of an accumulator register group are consecutive: their range planes
-      // come in 16-byte reads, requested together before the comparisons.  With one range the
-      // second range's planes hold the first's again (see request_scalars): the union is the same.
-      typedef int i32x4 __attribute__((ext_vector_type(4)));
+        for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
+      } else {
+        // the four queries of an accumulator register group are consecutive: their range planes
+        // come in 16-byte reads, requested together before the comparisons.  With one range the
+        // second range's planes hold the first's again (see request_scalars): the union is the same.
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          i32x4 rs[4];
+#pragma unroll
+          for (int pl = 0; pl < 4; ++pl) rs[pl] = *reinterpret_cast<const i32x4*>(&rng_lds[st][pl][QI * 32 + 8 * g + 4 * h]);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int s0 = rs[0][r], len0 = min(rs[1][r], seqlen_kv) - s0;
+            const int s1 = rs[2][r], len1 = min(rs[3][r], seqlen_kv) - s1;
+            bool ok = ((unsigned)(kv - s0) < (unsigned)max(len0, 0)) | ((unsigned)(kv - s1) < (unsigned)max(len1, 0));
+            ok &= qt * BM + QI * 32 + 8 * g + 4 * h + r < seqlen_q;
+            s_acc[4 * g + r] = ok ? 0.0f : -INFINITY;
+          }
+          __builtin_amdgcn_sched_barrier(0);  // one group's planes in registers at a time
+        }
+      }
+      // dP starts from -delta of its query (dS = P (dP - delta)): the subtraction rides on the
+      // accumulation instead of costing a vector instruction per element afterwards
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        i32x4 rs[4];
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][QI * 32 + 8 * g + 4 * h]);
 #pragma unroll
-        for (int pl = 0; pl < 4; ++pl) rs[pl] = *reinterpret_cast<const i32x4*>(&rng_lds[st][pl][qi * 32 + 8 * g + 4 * h]);
+        for (int r = 0; r < 4; ++r) dp_acc[4 * g + r] = d4[r];
+      }
+      // Everything the sub-step's 32 MFMAs read from LDS forms one stream, read AHEAD entries
+      // ahead into four rotating registers, across both matrix phases (the first operand of the
+      // second phase is on its way while the vector phase runs):
+      //   phase 1, per k-step: Q rows (-> S), [the parked V k-step (B operand)], dO rows (-> dP)
+      //   phase 2, per (16-query step s2, 32-dim block d): dO^T (-> dV), Q^T (-> dK)
+      constexpr int N1 = 2 * KS + VL, N2 = 4 * DT, NS = N1 + N2, AHEAD = 2, RING = 4, PRE = 1;
+      constexpr int FIRST_PARKED = 2 * (KS - VL);  // stream index of the first k-step with a parked V
+      auto entry = [&](int o) -> u32x4 {
+        if (o < N1) {
+          const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
+          const int kind = o < FIRST_PARKED ? (o & 1) * 2 : (o - FIRST_PARKED) % 3;  // 0: Q, 1: parked V, 2: dO
+          if (kind == 1) return v_park[w][VL > 0 ? ks - (KS - VL) : 0][lane];
+          return Tile::read_row(kind == 0 ? q_lds : do_lds, row_rd_q, 0, ks);
+        }
+        const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
+        return Tile::template read_col<true>((i & 1) ? q_lds : do_lds, col_rd_q, s2, d);
+      };
+      u32x4 buf[RING];
+#pragma unroll
+      for (int o = 0; o < AHEAD; ++o) buf[o] = entry(o);
+      // (after the step's first LDS reads are on their way: the requests are inline assembly that
+      // the compiler moves no memory access across)
+      if (QI == 0) request_scalars(head_next, qt_next, st ^ 1);
+#pragma unroll
+      for (int o = 0; o < N1; ++o) {
+        const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
+        const int kind = o < FIRST_PARKED ? (o & 1) * 2 : (o - FIRST_PARKED) % 3;
+        if (kind == 0) s_acc = mfma_32x32x16<DTYPE>(buf[o % RING], kreg[ks], s_acc);
+        else if (kind == 2 && ks < KS - VL) dp_acc = mfma_32x32x16<DTYPE>(buf[o % RING], vreg[ks < KS - VL ? ks : 0], dp_acc);
+        else if (kind == 2) dp_acc = mfma_32x32x16<DTYPE>(buf[o % RING], buf[(o - 1) % RING], dp_acc);
+        // the entry just used (and the one before it) are free: the next read goes there.  Only the
+        // first operand of the second phase is requested before the vector phase (registers)
+        if (o + AHEAD < N1 + PRE) buf[(o + AHEAD) % RING] = entry(o + AHEAD);
+        // this sub-step's half of the next step's tile loads, one per two k-steps
+        if (kind == 2 && ks % 2 == 0 && ks / 2 < NL / 2) request_tile(QI * (NL / 2) + ks / 2, head_next, qt_next, st ^ 1);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the order: reads neither pile up in registers nor fall behind
+      }
+      // ---- P = exp2(S c - lse), dS = P (dP - delta), packed in accumulator order: as B operands
+      // they feed the next products without leaving the registers -------------------------------
+      u32x4 pb[2], dsb[2];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int qrow = QI * 32 + 8 * g + 4 * h;
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[st][qrow]);
+        float pv[4], dsv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int s0 = rs[0][r], len0 = min(rs[1][r], seqlen_kv) - s0;
-          const int s1 = rs[2][r], len1 = min(rs[3][r], seqlen_kv) - s1;
-          bool ok = ((unsigned)(kv - s0) < (unsigned)max(len0, 0)) | ((unsigned)(kv - s1) < (unsigned)max(len1, 0));
-          ok &= qt * BM + qi * 32 + 8 * g + 4 * h + r < seqlen_q;
-          s_acc[4 * g + r] = ok ? 0.0f : -INFINITY;
+          pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));  // l4: lse * log2(e); masked: exp2(-inf) = 0
+          dsv[r] = pv[r] * dp_acc[4 * g + r];
         }
-        __builtin_amdgcn_sched_barrier(0);  // one group's planes in registers at a time
+        pb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(pv[0], pv[1]);
+        pb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(pv[2], pv[3]);
+        dsb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(dsv[0], dsv[1]);
+        dsb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(dsv[2], dsv[3]);
       }
-    }
-    // dP starts from -delta of its query (dS = P (dP - delta)): the subtraction rides on the
-    // accumulation instead of costing a vector instruction per element afterwards
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_lds[st][qi * 32 + 8 * g + 4 * h]);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) dp_acc[4 * g + r] = d4[r];
-    }
-    // Everything the step's 32 MFMAs read from LDS forms one stream, read AHEAD entries ahead
-    // into four rotating registers, across both matrix phases (the first operands of the second
-    // phase are on their way while the vector phase runs):
-    //   phase 1, per k-step: Q rows (-> S), [the parked V k-step (B operand)], dO rows (-> dP)
-    //   phase 2, per (16-query step s2, 32-dim block d): dO^T (-> dV), Q^T (-> dK)
-    constexpr int N1 = 2 * KS + VL, N2 = 4 * DT, NS = N1 + N2, AHEAD = 2;
-    constexpr int FIRST_PARKED = 2 * (KS - VL);  // stream index of the first k-step with a parked V
-    auto entry = [&](int o) -> u32x4 {
-      if (o < N1) {
-        const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
-        const int kind = o < FIRST_PARKED ? (o & 1) * 2 : (o - FIRST_PARKED) % 3;  // 0: Q, 1: parked V, 2: dO
-        if (kind == 1) return v_park[w][VL > 0 ? ks - (KS - VL) : 0][lane];
-        return Tile::read_row(kind == 0 ? q_lds : do_lds, row_rd, 0, ks);
-      }
-      const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
-      return Tile::template read_col<true>((i & 1) ? q_lds : do_lds, col_rd, s2, d);
-    };
-    u32x4 buf[4];
-#pragma unroll
-    for (int o = 0; o < AHEAD; ++o) buf[o] = entry(o);
-    // (after the step's first LDS reads are on their way: the requests are inline assembly that
-    // the compiler moves no memory access across)
-    request_scalars(head_next, qt_next, st ^ 1);
-#pragma unroll
-    for (int o = 0; o < N1; ++o) {
-      const int ks = o < FIRST_PARKED ? o / 2 : (KS - VL) + (o - FIRST_PARKED) / 3;
-      const int kind = o < FIRST_PARKED ? (o & 1) * 2 : (o - FIRST_PARKED) % 3;
-      if (kind == 0) s_acc = mfma_32x32x16<DTYPE>(buf[o & 3], kreg[ks], s_acc);
-      else if (kind == 2 && ks < KS - VL) dp_acc = mfma_32x32x16<DTYPE>(buf[o & 3], vreg[ks < KS - VL ? ks : 0], dp_acc);
-      else if (kind == 2) dp_acc = mfma_32x32x16<DTYPE>(buf[o & 3], buf[(o - 1) & 3], dp_acc);
-      // the entry just used (and the one before it) are free: the next read goes there.  Only the
-      // first operand of the second phase is requested before the vector phase (registers)
-      if (o + AHEAD <= N1) buf[(o + AHEAD) & 3] = entry(o + AHEAD);
-      if (kind == 2 && ks % 2 == 0 && ks / 2 < NL / 2) request_tile(ks / 2, head_next, qt_next, st ^ 1);
-      __builtin_amdgcn_sched_barrier(0);  // keeps the order: reads neither pile up in registers nor fall behind
-    }
-    // ---- P = exp2(S c - lse), dS = P (dP - delta), packed in accumulator order: as B operands
-    // they feed the next products without leaving the registers -------------------------------
-    u32x4 pb[2], dsb[2];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int qrow = qi * 32 + 8 * g + 4 * h;
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_lds[st][qrow]);
-      float pv[4], dsv[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pv[r] = fast_exp2(fmaf(s_acc[4 * g + r], p.scale_log2, -l4[r]));  // l4: lse * log2(e); masked: exp2(-inf) = 0
-        dsv[r] = pv[r] * dp_acc[4 * g + r];
-      }
-      pb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(pv[0], pv[1]);
-      pb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(pv[2], pv[3]);
-      dsb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(dsv[0], dsv[1]);
-      dsb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(dsv[2], dsv[3]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int o = N1 + 1; o < N1 + AHEAD; ++o) buf[o & 3] = entry(o);
-    // ---- dV^T[dim, key] += dO^T[dim, q] P[q, key];  dK^T[dim, key] += Q^T[dim, q] dS[q, key]
-    // over this wave's 32 queries (dO^T and Q^T come out of the row-major tiles by
-    // transpose loads, in the accumulators' row order) -----------------------------------------
-#pragma unroll
-    for (int o = N1; o < NS; ++o) {
-      const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
-      if (i & 1) dk_acc[d] = mfma_32x32x16<DTYPE>(buf[o & 3], dsb[s2], dk_acc[d]);
-      else dv_acc[d] = mfma_32x32x16<DTYPE>(buf[o & 3], pb[s2], dv_acc[d]);
-      if (o + AHEAD < NS) buf[(o + AHEAD) & 3] = entry(o + AHEAD);
-      constexpr int EVERY = N2 / (NL / 2);  // the second half of the tile loads, evenly over the phase
-      if ((i + 1) % EVERY == 0 && (i + 1) / EVERY <= NL / 2) request_tile(NL / 2 + (i + 1) / EVERY - 1, head_next, qt_next, st ^ 1);
       __builtin_amdgcn_sched_barrier(0);
-    }
+#pragma unroll
+      for (int o = N1 + PRE; o < N1 + AHEAD; ++o) buf[o % RING] = entry(o);
+      // ---- dV^T[dim, key] += dO^T[dim, q] P[q, key];  dK^T[dim, key] += Q^T[dim, q] dS[q, key]
+      // over the sub-step's 32 queries (dO^T and Q^T come out of the row-major tiles by
+      // transpose loads, in the accumulators' row order) ---------------------------------------
+#pragma unroll
+      for (int o = N1; o < NS; ++o) {
+        const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
+        if (i & 1) dk_acc[d] = mfma_32x32x16<DTYPE>(buf[o % RING], dsb[s2], dk_acc[d]);
+        else dv_acc[d] = mfma_32x32x16<DTYPE>(buf[o % RING], pb[s2], dv_acc[d]);
+        if (o + AHEAD < NS) buf[(o + AHEAD) % RING] = entry(o + AHEAD);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+#pragma clang loop unroll(disable)
+    for (int qi = 0; qi < 2; ++qi) sub_step(qi);
     st ^= 1;
     hg = hg_next;
   }
 
-  // ---- sum the two query halves: the qi = 0 waves finish dV, the qi = 1 waves dK; each
-  // wave hands the other product to its partner (same keys) through LDS ----------------------
-  wait_loads();     // the last step's (unused) requests have landed: the tile area is about to be reused
-  __syncthreads();  // nobody reads the tiles any more
-  float* red = reinterpret_cast<float*>(&tiles[0][0]) + w * (16 * DT * 64);
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) red[(dt * 16 + i) * 64 + lane] = qi == 0 ? dk_acc[dt][i] : dv_acc[dt][i];
-  __syncthreads();
-  const float* take = reinterpret_cast<const float*>(&tiles[0][0]) + (w ^ 2) * (16 * DT * 64);
-  const float out_scale = qi == 0 ? 1.0f : p.scale;
-  uint16_t* dst = reinterpret_cast<uint16_t*>(qi == 0 ? p.dv : p.dk);
+  // ---- dK and dV of the wave's keys are complete: scale, round, store ---------------------
+  wait_loads();  // the last step's (unused) requests must land before the workgroup's LDS is released
+  if (!has_keys) return;
   const int64_t off = (int64_t)p.dkv_block_table[(int64_t)b * p.max_kv_blocks + blk] * p.dkv_slot_stride +
-                      (int64_t)(tok0 + ki * 32 + c) * p.dkv_token_stride + (int64_t)kv_head * D + 4 * h;
+                      (int64_t)(tok0 + c) * p.dkv_token_stride + (int64_t)kv_head * D + 4 * h;
+  uint16_t* dv_dst = reinterpret_cast<uint16_t*>(p.dv) + off;
+  uint16_t* dk_dst = reinterpret_cast<uint16_t*>(p.dk) + off;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      float r[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        r[j] = ((qi == 0 ? dv_acc[dt][i] : dk_acc[dt][i]) + take[(dt * 16 + i) * 64 + lane]) * out_scale;
-      }
-      u32x2 v4 = {pack2<DTYPE>(r[0], r[1]), pack2<DTYPE>(r[2], r[3])};
-      *reinterpret_cast<u32x2*>(dst + off + dt * 32 + 8 * g) = v4;
+      const int i = 4 * g;
+      u32x2 v4 = {pack2<DTYPE>(dv_acc[dt][i], dv_acc[dt][i + 1]), pack2<DTYPE>(dv_acc[dt][i + 2], dv_acc[dt][i + 3])};
+      *reinterpret_cast<u32x2*>(dv_dst + dt * 32 + 8 * g) = v4;
+      u32x2 k4 = {pack2<DTYPE>(dk_acc[dt][i] * p.scale, dk_acc[dt][i + 1] * p.scale),
+                  pack2<DTYPE>(dk_acc[dt][i + 2] * p.scale, dk_acc[dt][i + 3] * p.scale)};
+      *reinterpret_cast<u32x2*>(dk_dst + dt * 32 + 8 * g) = k4;
     }
 }
 
@@ -697,8 +696,12 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
           s_acc = mfma_32x32x16<DTYPE>(ka[k4], qreg[half * 4 + k4], s_acc);
           dp_acc = mfma_32x32x16<DTYPE>(va[k4], doreg[half * 4 + k4], half == 0 && k4 == 0 ? dp_init : dp_acc);
         }
-        // one tile load per group of eight MFMAs: 2 * KS / 4 of the NL here, the rest below
-        if (nt * (KS / 4) + half < NL / 2) issue_load(nt * (KS / 4) + half);
+        // All of the tile's loads go out here, in the first phase, NL / (2 KS / 4) per group of
+        // eight MFMAs: the last one then has the whole dQ phase to land before the wait at the
+        // top of the next tile.
+        constexpr int PER = NL / (2 * (KS / 4));
+#pragma unroll
+        for (int l = 0; l < PER; ++l) issue_load((nt * (KS / 4) + half) * PER + l);
       }
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
@@ -727,10 +730,7 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) dq_acc[dt] = mfma_32x32x16<DTYPE>(kt_a[s2 & 1][dt], dsb[s2], dq_acc[dt]);
-      if (NL / 2 + s2 < NL) issue_load(NL / 2 + s2);
     }
-#pragma unroll
-    for (int i = NL / 2 + 4; i < NL; ++i) issue_load(i);
   };
 
   const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
@@ -839,18 +839,19 @@ extern "C" size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block
          align256(kTicketInts * sizeof(int32_t));
 }
 
-extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
-                            const void* out, const float* lse, void* dq, void* dk, void* dv,
-                            void* workspace, size_t workspace_bytes, const int32_t* cu_seqlens_q,
-                            const int32_t* cu_seqlens_kv, const int32_t* attn_range, int n_ranges,
-                            const int32_t* q_block_table, const int32_t* kv_block_table,
-                            const int32_t* out_block_table, const int32_t* dq_block_table,
-                            const int32_t* dkv_block_table, const int32_t* row_order, int batch,
-                            int max_kv_blocks, int total_q, int block_size, int n_heads_q,
-                            int n_heads_kv, int head_dim, int64_t kv_slot_stride,
-                            int64_t kv_token_stride, int64_t dkv_slot_stride,
-                            int64_t dkv_token_stride, int n_out_slots, float softmax_scale,
-                            int dtype, void* stream) {
+// Both entry points: argument checks, workspace carving, the four launches.
+static int attn_bwd_launch(const void* dout, const void* q, const void* k, const void* v,
+                           const void* out, const float* lse, void* dq, void* dk, void* dv,
+                           void* workspace, size_t workspace_bytes, const int32_t* cu_seqlens_q,
+                           const int32_t* cu_seqlens_kv, const int32_t* attn_range, int n_ranges,
+                           const int32_t* q_block_table, const int32_t* kv_block_table,
+                           const int32_t* out_block_table, const int32_t* dq_block_table,
+                           const int32_t* dkv_block_table, const int32_t* row_order, int batch,
+                           int max_kv_blocks, int total_q, int block_size, int n_heads_q,
+                           int n_heads_kv, int head_dim, int64_t kv_slot_stride,
+                           int64_t kv_token_stride, int64_t dkv_slot_stride,
+                           int64_t dkv_token_stride, int n_out_slots, float softmax_scale,
+                           int dtype, void* stream) {
   if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
     return fail(DCP_ERR_UNSUPPORTED, "attn_bwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
   if (head_dim != 64 && head_dim != 128)
@@ -923,7 +924,7 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
   p.n_out_slots = n_out_slots;
   p.q_tiles_per_row = (block_size + kBwdBM - 1) / kBwdBM;
   p.dq_tiles_per_row = (block_size + kDqBM - 1) / kDqBM;
-  p.kv_tiles_per_row = max_kv_blocks * (block_size / kBwdBN);
+  p.kv_tiles_per_row = (int)(((int64_t)max_kv_blocks * block_size + kDkvBN - 1) / kDkvBN);
   p.n_dkv_items = (int64_t)batch * n_heads_kv * p.kv_tiles_per_row;
   p.n_dq_items = (int64_t)batch * n_heads_q * p.dq_tiles_per_row;
   p.dkv_xcd_group = p.kv_tiles_per_row;
@@ -935,4 +936,23 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
                            : launch_bwd<DCP_DTYPE_BF16, 64>(p, (hipStream_t)stream);
   return head_dim == 128 ? launch_bwd<DCP_DTYPE_FP16, 128>(p, (hipStream_t)stream)
                          : launch_bwd<DCP_DTYPE_FP16, 64>(p, (hipStream_t)stream);
+}
+
+extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+                            const void* out, const float* lse, void* dq, void* dk, void* dv,
+                            void* workspace, size_t workspace_bytes, const int32_t* cu_seqlens_q,
+                            const int32_t* cu_seqlens_kv, const int32_t* attn_range, int n_ranges,
+                            const int32_t* q_block_table, const int32_t* kv_block_table,
+                            const int32_t* out_block_table, const int32_t* dq_block_table,
+                            const int32_t* dkv_block_table, const int32_t* row_order, int batch,
+                            int max_kv_blocks, int total_q, int block_size, int n_heads_q,
+                            int n_heads_kv, int head_dim, int64_t kv_slot_stride,
+                            int64_t kv_token_stride, int64_t dkv_slot_stride,
+                            int64_t dkv_token_stride, int n_out_slots, float softmax_scale,
+                            int dtype, void* stream) {
+  return attn_bwd_launch(dout, q, k, v, out, lse, dq, dk, dv, workspace, workspace_bytes, cu_seqlens_q,
+                         cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
+                         dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
+                         n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
+                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream);
 }

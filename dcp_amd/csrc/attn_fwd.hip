@@ -263,11 +263,13 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
   };
 
   // The tile loads of an iteration (this wave's share: LPW groups of K, LPW of V) are issued
-  // one at a time between the matrix instructions: as a burst after the barrier they fill the
-  // memory pipeline's queue and the wave sits at its last load until the queue has drained.
-  // They are issued unconditionally, so that the loop has no branches around them: past the
-  // end of the tile list the cursor stays on the last tile, which is then fetched again into
-  // a stage nobody reads any more.
+  // one at a time between the matrix instructions of the S^T product: as a burst after the
+  // barrier they fill the memory pipeline's queue and the wave sits at its last load until the
+  // queue has drained, and issued later (spread over the O^T product too) the last one is still
+  // on its way at the wait that opens the next iteration.  Both stages they fill are free from
+  // the iteration's first barrier on.  They are issued unconditionally, so that the loop has no
+  // branches around them: past the end of the tile list the cursor stays on the last tile,
+  // which is then fetched again into a stage nobody reads any more.
   constexpr int NL = 2 * KTile::LPW;
   uint32_t fill_k = 0, fill_v = 0;
   int64_t fill_k_off = 0, fill_v_off = 0;
@@ -310,7 +312,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
         s_out[i2 & 1][qb] = mfma_32x32x16<DTYPE>(ka[i2 & 3], qreg[qb][i2 >> 1], s_out[i2 & 1][qb]);
-      if ((i2 + 1) % (N / KTile::LPW) == 0) issue_load(i2 / (N / KTile::LPW));
+      if ((i2 + 1) % (N / NL) == 0) issue_load(i2 / (N / NL));
       __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from being hoisted into more registers
     }
   };
@@ -400,7 +402,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
           for (int c2 = lo; c2 < hi; ++c2) softmax_pair(sc, c2 / 16, c2 % 16);
         }
       }
-      if ((i + 1) % (N / KTile::LPW) == 0) issue_load(i / (N / KTile::LPW));
+      if ((i + 1) % (N / NL) == 0) issue_load(i / (N / NL));
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -420,7 +422,6 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
         o_acc[qb][i % DT] = mfma_32x32x16<DTYPE>(va[i & 3], pb[qb][i / DT], o_acc[qb][i % DT]);
-      if ((i + 1) % (N / VTile::LPW) == 0) issue_load(KTile::LPW + i / (N / VTile::LPW));
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -449,8 +450,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
     fill_v = v_fill;
     fill_k_off = cursor.off;
     fill_v_off = v_off;
-    // the S^T product carries the K loads, O^T += V^T P^T the V loads; a wave that skips one
-    // of them still has its share of the tile to request
+    // the S^T product carries the tile loads; a wave that skips it still has its share to request
     const bool nxt_full = j + 1 < n_tiles && tile_is_full(tile_nxt);
     bool cur = true;
     if (__builtin_expect(cur_full && nxt_full && anchored, 1)) {
@@ -486,7 +486,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
         multiply_qk(tile_nxt, k_nxt, s_nxt);
       } else {
 #pragma unroll
-        for (int i = 0; i < KTile::LPW; ++i) issue_load(i);
+        for (int i = 0; i < NL; ++i) issue_load(i);
       }
       if (cur) {
         if (!pending) softmax_max(s_cur);
@@ -500,9 +500,6 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
       __builtin_amdgcn_s_setprio(kPrioDense);
       multiply_pv(v_cur);
       __builtin_amdgcn_s_setprio(kPrioControl);
-    } else {
-#pragma unroll
-      for (int i = 0; i < VTile::LPW; ++i) issue_load(KTile::LPW + i);
     }
     cur_full = nxt_full;
     tile_cur = tile_nxt;
