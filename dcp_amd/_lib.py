@@ -36,6 +36,8 @@ SIGNATURES = {
     "dcp_attn_fwd_workspace_bytes": [],
     "dcp_attn_bwd": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
     "dcp_attn_bwd_workspace_bytes": [_I, _I, _I, _I, _I],
+    "dcp_attn_bwd_static": [_P] * 9 + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
+    "dcp_attn_bwd_static_scratch_bytes": [],
     "dcp_greedy_stage_selection": [_I, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P],
 }
 
@@ -70,7 +72,8 @@ def load():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = {"dcp_last_error": c_char_p, "dcp_attn_bwd_workspace_bytes": c_size_t,
-                          "dcp_attn_fwd_workspace_bytes": c_size_t}.get(name, c_int)
+                          "dcp_attn_fwd_workspace_bytes": c_size_t,
+                          "dcp_attn_bwd_static_scratch_bytes": c_size_t}.get(name, c_int)
         _lib = lib
     return _lib
 

@@ -956,3 +956,69 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
                          dkv_token_stride, n_out_slots, softmax_scale, dtype, stream);
 }
+
+// ---------------------------------------------------------------------------
+// The backward with its scratch inside the library, for callers that can neither allocate
+// nor pass a workspace.  Every device the library runs on holds its own copy of `scratch`
+// until the process ends.  In host code the array's name is only a handle: its device address
+// is asked for once per device (with that device current) and kept.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[DCP_ATTN_BWD_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device, or nullptr (message set).
+void* scratch_on_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(DCP_ERR_LAUNCH, "attn_bwd_static: no current device (or device index above %d)", kMaxDevices - 1);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      fail(DCP_ERR_LAUNCH, "attn_bwd_static: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+           hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" size_t dcp_attn_bwd_static_scratch_bytes(void) { return DCP_ATTN_BWD_STATIC_SCRATCH_BYTES; }
+
+extern "C" int dcp_attn_bwd_static(const void* dout, const void* q, const void* k, const void* v,
+                                   const void* out, const float* lse, void* dq, void* dk, void* dv,
+                                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_kv,
+                                   const int32_t* attn_range, int n_ranges, const int32_t* q_block_table,
+                                   const int32_t* kv_block_table, const int32_t* out_block_table,
+                                   const int32_t* dq_block_table, const int32_t* dkv_block_table,
+                                   const int32_t* row_order, int batch, int max_kv_blocks, int total_q,
+                                   int block_size, int n_heads_q, int n_heads_kv, int head_dim,
+                                   int64_t kv_slot_stride, int64_t kv_token_stride, int64_t dkv_slot_stride,
+                                   int64_t dkv_token_stride, int n_out_slots, float softmax_scale, int dtype,
+                                   void* stream) {
+  const size_t need = dcp_attn_bwd_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim);
+  DCP_REQUIRE(need <= (size_t)DCP_ATTN_BWD_STATIC_SCRATCH_BYTES,
+              "attn_bwd_static: these sizes need %zu bytes of scratch, the built-in scratch holds %zu; "
+              "use dcp_attn_bwd with a caller workspace",
+              need, (size_t)DCP_ATTN_BWD_STATIC_SCRATCH_BYTES);
+  void* ptr = scratch_on_current_device();
+  if (ptr == nullptr) return DCP_ERR_LAUNCH;
+  // Nothing in the scratch has to start at zero: delta, lse2 and the hulls are written for every
+  // valid (token, head) / query tile before the kernels that read them run (and only those are
+  // read), and the hull kernel zeroes the work counters on the stream.
+  return attn_bwd_launch(dout, q, k, v, out, lse, dq, dk, dv, ptr, DCP_ATTN_BWD_STATIC_SCRATCH_BYTES, cu_seqlens_q,
+                         cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
+                         dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
+                         n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
+                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream);
+}
+

@@ -267,6 +267,39 @@ size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
                                     int n_heads_q, int head_dim);
 
 /*
+ * dcp_attn_bwd for callers that cannot allocate device memory or carry a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Same arguments, results
+ * and errors as dcp_attn_bwd without `workspace`/`workspace_bytes`: the scratch
+ * is a static device array inside the library, DCP_ATTN_BWD_STATIC_SCRATCH_BYTES
+ * long, which every GPU the library runs on holds until the process ends (its
+ * address is looked up at the first call on a device).  The call allocates and
+ * frees nothing.  Sizes for which dcp_attn_bwd_workspace_bytes(...) exceeds the
+ * scratch are rejected with DCP_ERR_ARG.  All calls on one GPU share the one
+ * array: calls that may overlap on that GPU (different streams, or graphs
+ * replayed side by side) race; calls that follow each other on a stream do not.
+ */
+#define DCP_ATTN_BWD_STATIC_SCRATCH_BYTES (32u << 20)
+size_t dcp_attn_bwd_static_scratch_bytes(void);
+int dcp_attn_bwd_static(const void* dout, const void* q, const void* k,
+                        const void* v, const void* out, const float* lse,
+                        void* dq, void* dk, void* dv,
+                        const int32_t* cu_seqlens_q,
+                        const int32_t* cu_seqlens_kv,
+                        const int32_t* attn_range, int n_ranges,
+                        const int32_t* q_block_table,
+                        const int32_t* kv_block_table,
+                        const int32_t* out_block_table,
+                        const int32_t* dq_block_table,
+                        const int32_t* dkv_block_table,
+                        const int32_t* row_order, int batch, int max_kv_blocks,
+                        int total_q, int block_size, int n_heads_q,
+                        int n_heads_kv, int head_dim, int64_t kv_slot_stride,
+                        int64_t kv_token_stride, int64_t dkv_slot_stride,
+                        int64_t dkv_token_stride, int n_out_slots,
+                        float softmax_scale, int dtype, void* stream);
+
+/*
  * Stage packer of the planner (host code, no GPU work, `stream`-less): decides
  * which attention blocks ("workloads") every device may run in pipeline stage
  * `stage_id` and which data blocks must be sent to it first, under a cap on the
