@@ -79,6 +79,25 @@ def _kv_strides(k: torch.Tensor, v: torch.Tensor, name: str):
     return k.stride(0), k.stride(1)
 
 
+def _check_tables(batch, cu_seqlens_k, row_order, single, wide):
+    """The kernels index the block tables by row and, for the wide ones, with one common width:
+    a table of another shape would be read out of bounds or at the wrong slots."""
+    if cu_seqlens_k.numel() != batch + 1:
+        raise ValueError(f"cu_seqlens_k must have {batch + 1} entries like cu_seqlens_q, got {cu_seqlens_k.numel()}")
+    for name, t in single.items():
+        if tuple(t.shape) != (batch, 1):
+            raise ValueError(f"{name} must be [{batch}, 1], got {tuple(t.shape)}")
+    width = None
+    for name, t in wide.items():
+        if t.dim() != 2 or t.shape[0] != batch or t.shape[1] < 1:
+            raise ValueError(f"{name} must be [{batch}, max_blocks], got {tuple(t.shape)}")
+        if width is not None and t.shape[1] != width:
+            raise ValueError(f"{name} must have the width of kv_block_table ({width}), got {tuple(t.shape)}")
+        width = t.shape[1]
+    if row_order is not None and row_order.numel() != batch:
+        raise ValueError(f"row_order must have {batch} entries, got {row_order.numel()}")
+
+
 def _range_arg(attn_range: torch.Tensor, total_q: int):
     _i32(attn_range, "attn_range")
     if attn_range.dim() == 2 and tuple(attn_range.shape) == (2, total_q):
@@ -143,6 +162,8 @@ def _flash_attn_varlen_forward(
     kv_slot_stride, kv_token_stride = _kv_strides(k, v, "forward")
     n_ranges = _range_arg(attn_range, total_q)
     batch = cu_seqlens_q.numel() - 1
+    _check_tables(batch, cu_seqlens_k, row_order, dict(q_block_table=q_block_table, out_block_table=out_block_table),
+                  dict(kv_block_table=kv_block_table))
     if tuple(lse_.shape) != (n_heads_q, out_.shape[0], block_size):
         raise ValueError(f"lse_ shape {tuple(lse_.shape)} does not match out_")
     if softmax_scale is None:
@@ -207,8 +228,11 @@ def _flash_attn_varlen_backward(
     """Writes dQ into ``dq`` (slots ``dq_block_table``) and dK/dV into
     ``dk``/``dv`` (one slot per (row, kv block), ``dkv_block_table``).
     dK/dV of a kv head are summed over the q heads of its group inside the
-    kernel, and every token of a dK/dV slot is written, so ``dk``/``dv`` need
-    not be zeroed.
+    kernel, and the slots of a row's kv positions below its key count rounded up
+    to 32 are written whole (zeros where no query attends), so ``dk``/``dv`` need
+    not be zeroed when the key count is a multiple of the block size, as in
+    every plan.  Slot padding of q/k/v/out/dout may hold anything finite whose
+    dot products with the data stay finite; it is masked, not read as zero.
 
     ``workspace`` is scratch of ``backward_workspace_bytes(...)`` bytes (any
     dtype, contiguous); pass a preallocated tensor to keep the call
@@ -229,6 +253,9 @@ def _flash_attn_varlen_backward(
     dkv_slot_stride, dkv_token_stride = _kv_strides(dk, dv, "backward dk/dv")
     n_ranges = _range_arg(attn_range, total_q)
     batch = cu_seqlens_q.numel() - 1
+    _check_tables(batch, cu_seqlens_k, row_order,
+                  dict(q_block_table=q_block_table, out_block_table=out_block_table, dq_block_table=dq_block_table),
+                  dict(kv_block_table=kv_block_table, dkv_block_table=dkv_block_table))
     if softmax_lse.dtype != torch.float32 or not softmax_lse.is_contiguous():
         raise ValueError("softmax_lse must be contiguous float32")
     if tuple(softmax_lse.shape) != (n_heads_q, out.shape[0], block_size):

@@ -203,6 +203,11 @@ int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_offsets,
  * NULL = as numbered.  It changes no result.
  * Supported: dtype bf16/fp16, head_dim 64 or 128, block_size % 64 == 0,
  * softmax_scale > 0.
+ * Key/value tiles are loaded whole: what a slot holds past the row's keys (and,
+ * for keys a range excludes, inside it) reaches the matrix instructions and is
+ * masked there.  It must be finite, and small enough that its dot products with
+ * q stay finite; the reference's kernels zero-fill such loads instead.  Query
+ * rows past seqlen_q are not read.
  * `workspace`: caller-provided device scratch of at least
  * dcp_attn_fwd_workspace_bytes() bytes, 4-byte aligned, for the kernel's work
  * counters (the launch is persistent: its workgroups take (row, head, query
@@ -234,12 +239,18 @@ int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
  * dq ([n_dq_slots, block_size, n_heads_q, head_dim]) slot dq_block_table[b]
  * receives the row's dQ.  dk/dv: slot dkv_block_table[b*max_kv_blocks + j]
  * receives the dK/dV of the row's j-th kv block, summed over the q heads of
- * each kv head's group; every token of that slot is written (tokens no query
- * of the row attends get 0), so no pre-zeroing is needed.  No atomics are
- * used: results are bit-reproducible from run to run.
+ * each kv head's group.  The kv positions of the row below its key count
+ * (cu_seqlens_kv[b+1]-cu_seqlens_kv[b]) rounded up to 32 are written, all heads
+ * and dims, with 0 where no query of the row attends; positions past that keep
+ * what the slot held.  A key count that is a multiple of block_size, as every
+ * plan has it, therefore needs no pre-zeroing.  No atomics are used: results
+ * are bit-reproducible from run to run.
  * `workspace` is caller-provided device scratch of at least
  * dcp_attn_bwd_workspace_bytes(...) bytes, 16-byte aligned; its contents are
- * overwritten.  Key/value padding rows must hold finite values.
+ * overwritten.  Slot padding (q/dout/out rows past seqlen_q inside a 64-row
+ * tile, k/v rows past the row's keys) is loaded and masked, not skipped: it
+ * must be finite and small enough that its dot products with the data stay
+ * finite.
  */
 int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                  const void* out, const float* lse, void* dq, void* dk,

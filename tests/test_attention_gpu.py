@@ -2,29 +2,22 @@
 attention -> merge/scatter, and its backward) against the CPU oracle.
 
 Tolerances (bf16 inputs, fp32 accumulation, oracle in fp64 on the same rounded
-inputs): max-abs 2e-2 on outputs and gradients, 1e-3 on the fp32 LSE."""
+inputs): max-abs 2e-2 on out and dQ, max-abs 1e-3 on the fp32 LSE; dK/dV, which
+reach magnitudes where one bf16 ulp exceeds 2e-2, elementwise 2e-2 * max(1, |ref|)
+(tests/plan_cases.py)."""
 
 import numpy as np
 import pytest
 import torch
 
-from tests.plan_cases import dense_truth, make_case, run_executor, run_plan_oracle
+from tests.plan_cases import (LSE_TOL, OUT_TOL, check_against_truth, dense_truth, make_case, run_executor,
+                              run_plan_oracle)
 
 pytestmark = pytest.mark.gpu
 
-OUT_TOL = 2e-2
-LSE_TOL = 1e-3
 
-
-def _check_forward(case, res):
-    out, lse = res[0].float().numpy(), res[1].numpy()
-    t_out, t_lse = dense_truth(case)
-    assert np.isfinite(lse).all()
-    # absolute for |out| <= 1, relative above (one bf16 ulp exceeds the absolute bound from |out| = 4 on)
-    e_out = (np.abs(out - t_out) / np.maximum(1.0, np.abs(t_out))).max()
-    assert e_out <= OUT_TOL, e_out
-    e_lse = (np.abs(lse - t_lse) / np.maximum(1.0, np.abs(t_lse) / 16.0)).max()  # fp32 lse: ~1e-7 relative
-    assert e_lse <= LSE_TOL, e_lse
+def _check_forward(case, res, out_tol=OUT_TOL):
+    check_against_truth(res[:2], dense_truth(case), out_tol)
 
 
 FWD_CASES = {
@@ -74,11 +67,18 @@ FWD_CASES = {
 }
 
 
+# With inputs three times the usual size an output element reaches 13 in magnitude, where the
+# output type's own spacing is 2^-4 (bf16, from 8 on): a result rounded correctly can be 3.1e-2
+# away from the truth, so that case (bf16) allows one such step, 6.25e-2.  Every other case holds
+# the plain 2e-2.
+WIDE_OUT = {"large_scores": 6.25e-2}
+
+
 @pytest.mark.parametrize("name", list(FWD_CASES))
 def test_forward_matches_dense_truth(gpu, name):
     case = make_case(**FWD_CASES[name])
     res, _ = run_executor(case)
-    _check_forward(case, res)
+    _check_forward(case, res, WIDE_OUT.get(name, OUT_TOL))
 
 
 def test_forward_matches_plan_oracle_buffers(gpu):
@@ -89,16 +89,6 @@ def test_forward_matches_plan_oracle_buffers(gpu):
     ref = run_plan_oracle(case)
     assert np.abs(res[0].float().numpy() - ref[0].float().numpy()).max() <= OUT_TOL
     assert np.abs(res[1].numpy() - ref[1].numpy()).max() <= LSE_TOL
-
-
-GRAD_ATOL = 2e-2
-GRAD_RTOL = 2e-2  # gradients of long rows exceed 1 in magnitude: 2e-2 * max(1, |ref|)
-
-
-def _grad_err(got, ref):
-    """Largest |got - ref| / max(1, |ref|)."""
-    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
-    return float((np.abs(got - ref) / np.maximum(1.0, np.abs(ref))).max())
 
 
 BWD_CASES = {
@@ -127,12 +117,7 @@ BWD_CASES = {
 def test_backward_matches_dense_truth(gpu, name):
     case = make_case(**BWD_CASES[name])
     res, _ = run_executor(case, backward=True)
-    _check_forward(case, res)
-    _, _, t_dq, t_dkv = dense_truth(case, backward=True)
-    e_dq = _grad_err(res[2].float().numpy(), t_dq)
-    e_dkv = _grad_err(res[3].float().numpy(), t_dkv)
-    assert e_dq <= GRAD_ATOL, e_dq
-    assert e_dkv <= GRAD_ATOL, e_dkv
+    check_against_truth(res, dense_truth(case, backward=True))
 
 
 def test_forward_workspace_is_reusable_and_may_hold_anything(gpu):

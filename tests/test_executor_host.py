@@ -62,3 +62,25 @@ def test_synchronize_must_be_registered():
         ex.execute(_plan([m]))
     with pytest.raises(NotImplementedError):
         DCPExecutor()._create_buffer((1,), 0)
+
+
+def test_attention_wrappers_reject_block_tables_of_the_wrong_shape():
+    """The kernels index every wide table with kv_block_table's width and every table by row:
+    a mismatch is a ValueError on the host, not an out-of-bounds read on the device."""
+    import torch
+
+    from dcp_amd.flash_attn_interface import _check_tables
+
+    i32 = lambda *shape: torch.zeros(*shape, dtype=torch.int32)
+    ok = dict(q_block_table=i32(3, 1), out_block_table=i32(3, 1))
+    _check_tables(3, i32(4), None, ok, dict(kv_block_table=i32(3, 5), dkv_block_table=i32(3, 5)))
+    with pytest.raises(ValueError, match="width of kv_block_table"):
+        _check_tables(3, i32(4), None, ok, dict(kv_block_table=i32(3, 5), dkv_block_table=i32(3, 8)))
+    with pytest.raises(ValueError, match=r"q_block_table must be \[3, 1\]"):
+        _check_tables(3, i32(4), None, dict(q_block_table=i32(4, 1)), dict(kv_block_table=i32(3, 5)))
+    with pytest.raises(ValueError, match="kv_block_table must be"):
+        _check_tables(3, i32(4), None, ok, dict(kv_block_table=i32(2, 5)))
+    with pytest.raises(ValueError, match="cu_seqlens_k"):
+        _check_tables(3, i32(5), None, ok, dict(kv_block_table=i32(3, 5)))
+    with pytest.raises(ValueError, match="row_order"):
+        _check_tables(3, i32(4), i32(2), ok, dict(kv_block_table=i32(3, 5)))

@@ -21,6 +21,7 @@ import torch
 
 import bench
 from oracle import dcp_oracle as oracle
+from tests.plan_cases import max_abs_err, scaled_err
 
 pytestmark = pytest.mark.gpu
 
@@ -67,11 +68,11 @@ def _sample_check(wl, layout, mask, t, samples):
         q, dout = np.concatenate(qs, axis=1), np.concatenate(douts, axis=1)
         m = mask[int(seq_off[s]) : int(seq_off[s]) + L].numpy()
         r_out, r_lse, r_dq, r_dkv = oracle.dense_reference(q, kv, m, [L], dout=dout, dtype=np.float64)
-        rel = lambda g, r: float((np.abs(g - r) / np.maximum(1.0, np.abs(r))).max())
-        worst["out"] = max(worst["out"], rel(np.concatenate(outs, axis=1), r_out))
-        worst["lse"] = max(worst["lse"], float(np.abs(np.concatenate(lses, axis=0) - r_lse).max()))
-        worst["dq"] = max(worst["dq"], rel(np.concatenate(dqs, axis=1), r_dq))
-        worst["dkv"] = max(worst["dkv"], rel(t[B.LOCAL_dKV][sl_kv].float().cpu().numpy(), r_dkv))
+        # max-abs for out, LSE and dQ; dK/dV (magnitudes far above 1 at these lengths) scaled by max(1, |ref|)
+        worst["out"] = max(worst["out"], max_abs_err(np.concatenate(outs, axis=1), r_out))
+        worst["lse"] = max(worst["lse"], max_abs_err(np.concatenate(lses, axis=0), r_lse))
+        worst["dq"] = max(worst["dq"], max_abs_err(np.concatenate(dqs, axis=1), r_dq))
+        worst["dkv"] = max(worst["dkv"], scaled_err(t[B.LOCAL_dKV][sl_kv].float().cpu().numpy(), r_dkv))
     return worst
 
 
@@ -97,7 +98,8 @@ def _dense_check_gpu(wl, mask, t, s, kvh, chunk=4096):
     dk = torch.zeros(L, d, dtype=torch.float64, device="cuda")
     dv = torch.zeros_like(dk)
     worst = dict(out=0.0, lse=0.0, dq=0.0, dkv=0.0)
-    rel = lambda g, r: float(((g - r).abs() / r.abs().clamp(min=1.0)).max())
+    rel = lambda g, r: float(((g - r).abs() / r.abs().clamp(min=1.0)).max())  # dK/dV only
+    mabs = lambda g, r: float((g - r).abs().max())
     hblk, n_hblk = kvh * group // hb, max(1, group // hb)
     for j in range(n_hblk):
         sl = slice((hblk + j) * total + o0, (hblk + j) * total + o0 + L)
@@ -118,9 +120,9 @@ def _dense_check_gpu(wl, mask, t, s, kvh, chunk=4096):
                 dk += (ds.T @ q[r0:r1]) * scale
                 dv += pr.T @ do[r0:r1]
                 rs = slice(sl.start + r0, sl.start + r1)
-                worst["out"] = max(worst["out"], rel(t[B.LOCAL_OUT][rs, hh].double(), out))
+                worst["out"] = max(worst["out"], mabs(t[B.LOCAL_OUT][rs, hh].double(), out))
                 worst["lse"] = max(worst["lse"], float((t[B.LOCAL_LSE][hh, rs].double() - lse).abs().max()))
-                worst["dq"] = max(worst["dq"], rel(t[B.LOCAL_dQ][rs, hh].double(), dq))
+                worst["dq"] = max(worst["dq"], mabs(t[B.LOCAL_dQ][rs, hh].double(), dq))
     got = t[B.LOCAL_dKV][kvh * total + o0 : kvh * total + o0 + L].double()
     worst["dkv"] = max(rel(got[:, 0, 0], dk), rel(got[:, 1, 0], dv))
     return worst
@@ -235,9 +237,12 @@ def test_config2_split_over_four_devices_matches_one_device(gpu):
     torch.cuda.synchronize()
     dq = sum(lay.from_local_q(ex.buffers[B.LOCAL_dQ]) for lay, ex in zip(lays, exs))
     dkv = sum(lay.from_local_kv(ex.buffers[B.LOCAL_dKV]) for lay, ex in zip(lays, exs))
-    for got, want in ((dq, one["dq"]), (dkv, one["dkv"])):
-        err = (got.float() - want.float()).abs()
-        assert bool((err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * float(want.float().abs().max())).all())
+    # two bf16 results against each other (here the partial gradients also travel in bf16): dQ max-abs,
+    # dK/dV scaled by max(1, |want|) as everywhere
+    e_dq = float((dq.float() - one["dq"].float()).abs().max())
+    e_dkv = float(((dkv.float() - one["dkv"].float()).abs() / one["dkv"].float().abs().clamp(min=1.0)).max())
+    print("four devices vs one: dq", e_dq, "dkv (scaled)", e_dkv, flush=True)
+    assert e_dq <= 2e-2 and e_dkv <= 2e-2, (e_dq, e_dkv)
 
 
 def test_config3_lambda_mask_sampled_parity(gpu):
