@@ -101,7 +101,31 @@ __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
   float row_lse[TPG];  // the same in every iteration over w: it only depends on the LSEs
 #pragma unroll
   for (int k = 0; k < TPG; ++k) row_lse[k] = -1.0f;
-  for (int w = g; w < n_words; w += lanes_per_row) {
+  // An op with a single source is the scatter-back of a finished block: its finite rows are
+  // copied bit for bit (the weighted sum 0 + 1 * x would turn -0.0 into +0.0).
+  const bool copy_only = n_src == 1;
+  for (int w = g; copy_only && w < n_words; w += lanes_per_row) {
+    const int64_t blk = table[0];
+#pragma unroll
+    for (int k = 0; k < TPG; ++k) {
+      const float l = lse_head[t[k] * lse_token_stride + blk * lse_block_stride];
+      const raw* p = out_head + t[k] * out_token_stride + blk * out_block_stride + (int64_t)w * VN;
+      const bool finite = lse_is_finite(l);
+      row_lse[k] = finite ? l : -1.0f;
+      if (!live[k]) continue;
+      const int64_t dst_tok = (int64_t)dst_token_offsets[op] + t[k];
+      raw* q = dst_out + dst_tok * out_token_stride + (int64_t)h * head_dim + (int64_t)w * VN;
+      if constexpr (VECTOR) {
+        u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        const u32x4 zero = {0, 0, 0, 0};
+        __builtin_nontemporal_store(finite ? x : zero, reinterpret_cast<u32x4*>(q));
+      } else {
+        const raw x = *p;
+        *q = finite ? x : Elem<DTYPE>::store(0.0f);
+      }
+    }
+  }
+  for (int w = g; !copy_only && w < n_words; w += lanes_per_row) {
     float m[TPG], ssum[TPG], acc[TPG][VN];
 #pragma unroll
     for (int k = 0; k < TPG; ++k) {
@@ -270,7 +294,15 @@ __global__ __launch_bounds__(256) void blockwise_sum_kernel(
 #pragma unroll
       for (int k = 0; k < VN; ++k) acc[u][k] = 0.0f;
     }
-    if (begin < vec_end) {
+    if (begin < vec_end && n_ops == 1) {  // a single source: the scatter-back, copied bit for bit
+      const raw* row = src + offs[0] * src_stride;
+      u32x4 bits[kSumUnroll];
+#pragma unroll
+      for (int u = 0; u < kSumUnroll; ++u) bits[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + pos[u]));
+#pragma unroll
+      for (int u = 0; u < kSumUnroll; ++u)
+        if (live[u]) __builtin_nontemporal_store(bits[u], reinterpret_cast<u32x4*>(dst + pos[u]));
+    } else if (begin < vec_end) {
       for (int j0 = 0; j0 < n_ops; j0 += 4) {
         u32x4 bits[4][kSumUnroll];
 #pragma unroll
@@ -293,6 +325,10 @@ __global__ __launch_bounds__(256) void blockwise_sum_kernel(
     }
   }
   for (int64_t i = vec_end + threadIdx.x; i < end; i += 256) {
+    if (n_ops == 1) {
+      dst[i] = src[offs[0] * src_stride + i];
+      continue;
+    }
     float acc = 0.0f;
     for (int j = 0; j < n_ops; ++j) acc += Elem<DTYPE>::load(src[offs[j] * src_stride + i]);
     dst[i] = Elem<DTYPE>::store(acc);

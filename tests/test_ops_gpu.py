@@ -61,14 +61,14 @@ def test_fused_copy_full_blocks_and_unaligned(gpu):
     torch.cuda.synchronize()
     expect = torch.zeros_like(src)
     expect[[1, 3, 4]] = src[[5, 0, 2]]
-    assert torch.equal(dst, expect)
+    assert torch.equal(dst.view(torch.int16), expect.view(torch.int16))
     # source and destination misaligned by one element (2 bytes)
     dst.zero_()
     fused_copy_bf16_varlen(i64([src.data_ptr() + 2]), i32([0]), i32([1]), i64([dst.data_ptr() + 6]),
                            i32([0]), i32([1]), i32([777]), 4096, 128)
     torch.cuda.synchronize()
     flat_s, flat_d = src.reshape(-1), dst.reshape(-1)
-    assert torch.equal(flat_d[3:780], flat_s[1:778])
+    assert torch.equal(flat_d[3:780].view(torch.int16), flat_s[1:778].view(torch.int16))
     assert flat_d[:3].abs().sum() == 0 and flat_d[780:].abs().sum() == 0
 
 
@@ -89,7 +89,7 @@ def test_fused_copy_dkv_bit_exact(gpu):
         torch.tensor([dst[d].data_ptr() for d in dst_idx], dtype=torch.int64, device=gpu),
         torch.tensor(n_tokens, dtype=torch.int32, device=gpu), max_tokens, per_token, 128)
     torch.cuda.synchronize()
-    assert torch.equal(dst, expect)
+    assert torch.equal(dst.view(torch.int16), expect.view(torch.int16))
 
 
 @pytest.mark.parametrize("heads", [1, 4, 5])
@@ -114,7 +114,7 @@ def test_fused_copy_lse_bit_exact(gpu, heads):
                                i64([dst.data_ptr()] * k), i32([s * bs for s in slots]),
                                i32([n_slots * bs] * k), i32(n_tokens), heads, bs, 128)
     torch.cuda.synchronize()
-    assert torch.equal(dst, expect)
+    assert torch.equal(dst.view(torch.int32), expect.view(torch.int32))
 
 
 def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, inf_frac=0.0,
@@ -202,6 +202,61 @@ def test_update_out_lse_single_source_is_exact_copy(gpu):
     assert err_out == 0.0 and err_lse == 0.0
 
 
+@pytest.mark.parametrize("name", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("width", [1, 4])
+def test_single_source_merge_and_sum_copy_bit_patterns(gpu, name, width):
+    """Ops with one source are the scatter-back of finished blocks: bit for bit the source,
+    negative zeros and NaN payloads included (compared as integers, not as floats), also when
+    the launch's table is wide enough for more sources; a source whose LSE is infinite gives
+    zeros and LSE -1."""
+    from dcp_amd.ops.fused_ops import flash_attn_update_out_lse, fused_blockwise_sum
+
+    dtype = DTYPES[name]
+    ibits = torch.int32 if dtype == torch.float32 else torch.int16
+    g = torch.Generator().manual_seed(9)
+    bs, heads, d, n_blocks = 128, 3, 64, 5
+    src = torch.randn(n_blocks, bs, heads, d, generator=g).to(dtype)
+    flat = src.view(ibits).reshape(-1)
+    sign = torch.tensor(-0.0, dtype=dtype).view(ibits)  # the sign bit alone = -0.0
+    nan = torch.tensor(float("nan"), dtype=dtype).view(ibits) | 5  # a NaN with a payload
+    flat[::7] = sign
+    flat[3::11] = nan
+    lse = torch.randn(heads, n_blocks, bs, generator=g)
+    lse.view(torch.int32).reshape(-1)[::13] |= -2147483648  # some negative LSEs, sign set by bit
+    lse[1, 2, 5] = float("inf")
+    lse[2, 4, 7] = float("-inf")
+    n_tok = [bs, 1, 77]
+    blocks = [4, 0, 2]
+    offs = [0, bs, bs + 1]
+    total = sum(n_tok)
+    i32 = lambda v: torch.tensor(np.asarray(v), dtype=torch.int32, device=gpu)
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device=gpu)
+    table = [[b] + [-1] * (width - 1) for b in blocks]
+    d_src, d_lse = src.to(gpu), lse.to(gpu)
+    dst_out = torch.ones(total, heads, d, dtype=dtype, device=gpu)
+    dst_lse = torch.ones(heads, total, device=gpu)
+    flash_attn_update_out_lse(d_src, dst_out, d_lse, dst_lse, heads, i32(table), i32(offs), i32(n_tok), i32([1] * 3), bs,
+                              bs * heads * d, heads * d, bs, 1, n_blocks * bs, total, d, width, 64)
+    torch.cuda.synchronize()
+    for b, o, n in zip(blocks, offs, n_tok):
+        want_out, want_lse = src[b, :n].clone(), lse[:, b, :n].clone()
+        dead = ~torch.isfinite(want_lse)  # [heads, n]
+        want_out[dead.T] = 0.0
+        want_lse[dead] = -1.0
+        assert torch.equal(dst_out[o : o + n].cpu().view(ibits), want_out.view(ibits))
+        assert torch.equal(dst_lse[:, o : o + n].cpu().view(torch.int32), want_lse.view(torch.int32))
+    # the block sum with one source per sum
+    numel = bs * heads * d
+    dst = torch.ones(n_blocks, bs, heads, d, dtype=dtype, device=gpu)
+    dst_idx = [1, 3, 0]
+    fused_blockwise_sum(i64([d_src.data_ptr()] * 3), i32(table), i32([numel] * 3), i32([1] * 3), i64([dst.data_ptr()] * 3),
+                        i32(dst_idx), i32([numel] * 3), i32([n * heads * d for n in n_tok]), dtype, width, numel, 128)
+    torch.cuda.synchronize()
+    for b, di, n in zip(blocks, dst_idx, n_tok):
+        assert torch.equal(dst[di, :n].cpu().view(ibits), src[b, :n].view(ibits))
+        assert bool((dst[di, n:] == 1).all())
+
+
 def test_update_out_lse_rejects_too_many_sources(gpu):
     from dcp_amd.ops.fused_ops import flash_attn_update_out_lse
 
@@ -221,6 +276,7 @@ def test_fused_blockwise_sum(gpu, name, tol):
     block_size, n_blocks, n_heads, head_dim, max_ops, n_reds = 512, 64, 2, 64, 8, 8
     src = torch.randn(n_blocks, block_size, n_heads, head_dim, generator=g).to(dtype).to(gpu)
     dst = torch.randn(n_blocks, block_size, n_heads, head_dim, generator=g).to(dtype).to(gpu)
+    before = dst.clone()
     ops_per_red = rng.integers(1, max_ops + 1, n_reds)
     ops_per_red[0] = 1
     red_blocks = rng.choice(n_blocks, int(ops_per_red.sum()), replace=False)
@@ -245,12 +301,12 @@ def test_fused_blockwise_sum(gpu, name, tol):
     torch.cuda.synchronize()
     got = dst.float().cpu().numpy()
     assert np.abs(got - expect).max() <= tol
-    # single-source sums are exact copies
-    d0, n0 = dst_idx[0], n_tok[0]
-    assert np.array_equal(got[d0, :n0], src_np[lists[0][0], :n0])
-    # untouched blocks stay bit-identical
+    # single-source sums are copies, and untouched blocks stay as they were: compared as integers
+    ibits = torch.int32 if dtype == torch.float32 else torch.int16
+    d0, n0 = int(dst_idx[0]), int(n_tok[0])
+    assert torch.equal(dst[d0, :n0].view(ibits), src[int(lists[0][0]), :n0].view(ibits))
     untouched = sorted(set(range(n_blocks)) - set(dst_idx.tolist()))
-    assert np.array_equal(got[untouched], expect[untouched])
+    assert torch.equal(dst[untouched].view(ibits).cpu(), before[untouched].view(ibits).cpu())
 
 
 def test_fused_blockwise_sum_rejects_dtype(gpu):
