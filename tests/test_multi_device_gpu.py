@@ -6,9 +6,20 @@ import numpy as np
 import pytest
 import torch
 
-from tests.plan_cases import dense_truth, make_multi_case, run_multi_executor, run_multi_oracle
+from tests.plan_cases import (dense_truth, make_multi_case, max_abs_err, run_multi_executor, run_multi_oracle,
+                              scaled_err)
 
 pytestmark = pytest.mark.gpu
+
+
+def _grads_close(dq, dkv, want_dq, want_dkv):
+    """max-abs 2e-2 on dQ.  dK/dV: 4e-2 * max(1, |ref|), twice the one-device bound of
+    tests/plan_cases.py: here every device rounds its partial dK/dV to bf16 before the owner adds
+    them (inputs are unscaled N(0,1), so elements reach 10 and more), one rounding more than on one
+    device; measured worst case 2.9e-2."""
+    e_dq = max_abs_err(dq.float().numpy(), np.asarray(want_dq, dtype=np.float64) if not torch.is_tensor(want_dq) else want_dq.float().numpy())
+    e_dkv = scaled_err(dkv.float().numpy(), np.asarray(want_dkv, dtype=np.float64) if not torch.is_tensor(want_dkv) else want_dkv.float().numpy())
+    assert e_dq <= 2e-2 and e_dkv <= 4e-2, (e_dq, e_dkv)
 
 CASES = {
     "two_devices_causal": dict(n_nodes=1, n_devices_per_node=2, seqlens=[200, 330], block_size=64, n_heads=4,
@@ -33,9 +44,8 @@ def test_exchange_matches_oracle_and_dense_attention(name):
         assert (got.float() - want.float()).abs().max() <= 2e-2
     for want in (o_lse, torch.from_numpy(t_lse)):
         assert (lse.float() - want.float()).abs().max() <= 1e-3
-    for got, want in ((dq, torch.from_numpy(t_dq)), (dkv, torch.from_numpy(t_dkv)), (dq, o_dq), (dkv, o_dkv)):
-        err = (got.float() - want.float()).abs()
-        assert (err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * want.float().abs().max()).all()
+    _grads_close(dq, dkv, t_dq, t_dkv)
+    _grads_close(dq, dkv, o_dq, o_dkv)
 
 
 def test_exchange_can_be_repeated():
@@ -190,9 +200,7 @@ def test_random_placements_against_oracle(seed):
     o_out, o_lse, o_dq, o_dkv = run_multi_oracle(case, backward=True)
     assert (out.float() - o_out.float()).abs().max() <= 2e-2
     assert (lse.float() - o_lse.float()).abs().max() <= 1e-3
-    for got, want in ((dq, o_dq), (dkv, o_dkv)):
-        err = (got.float() - want.float()).abs()
-        assert (err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * want.float().abs().max()).all()
+    _grads_close(dq, dkv, o_dq, o_dkv)
 
 
 STAGED = {
@@ -220,9 +228,8 @@ def test_staged_exchange_matches_oracle_and_dense_attention(name):
         assert (out.float() - want.float()).abs().max() <= 2e-2
     for want in (o_lse, torch.from_numpy(t_lse)):
         assert (lse.float() - want.float()).abs().max() <= 1e-3
-    for got, want in ((dq, torch.from_numpy(t_dq)), (dkv, torch.from_numpy(t_dkv)), (dq, o_dq), (dkv, o_dkv)):
-        err = (got.float() - want.float()).abs()
-        assert (err <= 2e-2 * want.float().abs().clamp(min=1.0) + 4e-3 * want.float().abs().max()).all()
+    _grads_close(dq, dkv, t_dq, t_dkv)
+    _grads_close(dq, dkv, o_dq, o_dkv)
 
 
 def test_a_device_that_sends_to_itself_runs_through_plain_execute():
