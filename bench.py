@@ -169,6 +169,39 @@ def time_steps(ex_f, ex_b, fw, bw, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+_PROBES = None
+
+
+def load_probes():
+    """libbench_probes.so (bench_probes.hip, built by `python -m dcp_amd.build`): the two
+    measurement-only kernels this benchmark runs beside the product library."""
+    global _PROBES
+    if _PROBES is None:
+        import ctypes
+
+        import torch  # noqa: F401  (first: one HIP runtime per process)
+
+        path = os.path.join(ROOT, "libbench_probes.so")
+        if not os.path.exists(path):
+            raise SystemExit(f"{path} is not built; run `python -m dcp_amd.build`")
+        lib = ctypes.CDLL(path)
+        P, I = ctypes.c_void_p, ctypes.c_int
+        lib.bench_mfma_probe.argtypes = [P, P, I, I, I, P, P]
+        lib.bench_hbm_stream_probe.argtypes = [P, P, I, ctypes.c_size_t, P]
+        lib.bench_probe_last_error.restype = ctypes.c_char_p
+        _PROBES = lib
+    return _PROBES
+
+
+def call_probe(name, *args):
+    """Status 1 (argument) -> AssertionError, 2 (unsupported) -> ValueError, as the product library's calls."""
+    lib = load_probes()
+    status = getattr(lib, name)(*args)
+    if status != 0:
+        message = f"{name}: {lib.bench_probe_last_error().decode(errors='replace')}"
+        raise {1: AssertionError, 2: ValueError}.get(status, RuntimeError)(message)
+
+
 def mfma_sustained(iters=60000):
     """What the matrix cores sustain on this device when a kernel does nothing but bf16
     32x32x16 MFMAs, one wave per SIMD: with constant operands (full shader clock) and with
@@ -178,7 +211,6 @@ def mfma_sustained(iters=60000):
     import ctypes
 
     import torch
-    from dcp_amd import _lib
 
     n_wg = torch.cuda.get_device_properties(0).multi_processor_count
     n_words = n_wg * 256 * 16 * 8  # 16 x 16 bytes per thread, as bf16
@@ -191,10 +223,10 @@ def mfma_sustained(iters=60000):
                else torch.randn(n_words, device="cuda", generator=g)).to(torch.bfloat16)
         flop = ctypes.c_double()
         args = (ops.data_ptr(), out.data_ptr(), n_wg, iters, 0, ctypes.byref(flop), stream)
-        _lib.call("dcp_mfma_probe", *args)  # warm-up
+        call_probe("bench_mfma_probe", *args)  # warm-up
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        _lib.call("dcp_mfma_probe", *args)
+        call_probe("bench_mfma_probe", *args)
         e1.record()
         torch.cuda.synchronize()
         clocks, ticks = out[:2].tolist()
@@ -225,7 +257,7 @@ def movement_microbench(iters=5, bs=512):
     4-way (out, lse) merge.  Returns GB/s from events on the launch stream."""
     import torch
     from dcp_amd import _lib
-    from dcp_amd.ops.fused_ops import flash_attn_update_out_lse, fused_copy_bf16_varlen
+    from dcp_amd.ops.fused_ops import flash_attn_update_out_lse, fused_blockwise_sum, fused_copy_bf16_varlen
 
     tokens, heads, d = 262144, 32, 128
     n_blocks = tokens // bs
@@ -277,13 +309,27 @@ def movement_microbench(iters=5, bs=512):
     merge_bytes = (n_src + 1) * (d * 2 + 4) * tokens * heads
     merge_gbps = merge_bytes / (total / n * 1e-3) / 1e9
 
+    # block sum: the same four sources per block added up (fp32 accumulation, one rounding)
+    sum_args = (i64([outs.data_ptr()] * n_blocks), table, stride, i32([n_src] * n_blocks), i64([dst_out.data_ptr()] * n_blocks),
+                i32(ident), stride, full, torch.bfloat16, n_src, numel, 128)
+    fused_blockwise_sum(*sum_args)
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    for _ in range(iters):
+        fused_blockwise_sum(*sum_args)
+    torch.cuda.synchronize()
+    _lib.profile_enable(False)
+    n, total = _lib.profile_report()["blockwise_sum_kernel"]
+    sum_bytes = (n_src + 1) * tokens * heads * d * 2
+    sum_gbps = sum_bytes / (total / n * 1e-3) / 1e9
+
     # what a plain streaming kernel reaches at the same read : write mixes on the same buffers
     # (1 read + 1 write like the copy, 4 reads + 1 write like the merge): the practical ceiling
     stream_gbps = {}
     stream = torch.cuda.current_stream().cuda_stream
     per_stream = tokens * heads * d * 2  # 2 GiB
     for ns in (1, 4):
-        call = lambda: _lib.call("dcp_hbm_stream_probe", outs.data_ptr(), dst_out.data_ptr(), ns, per_stream, stream)
+        call = lambda: call_probe("bench_hbm_stream_probe", outs.data_ptr(), dst_out.data_ptr(), ns, per_stream, stream)
         call()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -301,6 +347,9 @@ def movement_microbench(iters=5, bs=512):
         merge4_GBps=round(merge_gbps, 1),
         merge4_frac_of_8TBps=round(merge_gbps / PEAK_HBM_GBPS, 4),
         merge_bytes_per_launch=merge_bytes,
+        block_sum4_GBps=round(sum_gbps, 1),
+        block_sum4_frac_of_8TBps=round(sum_gbps / PEAK_HBM_GBPS, 4),
+        block_sum_bytes_per_launch=sum_bytes,
         plain_stream_1r1w_GBps=round(stream_gbps[1], 1),
         plain_stream_4r1w_GBps=round(stream_gbps[4], 1),
     )
@@ -376,12 +425,13 @@ def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
     ``budget_s`` seconds of CPU work are done."""
     from oracle import dcp_oracle as oracle
 
-    try:
-        from threadpoolctl import threadpool_info
+    # the threads the oracle's matrix products really run on (numpy's BLAS pool); no silent default
+    from threadpoolctl import threadpool_info
 
-        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
-    except Exception:
-        threads = 1
+    pools = [p["num_threads"] for p in threadpool_info() if p.get("user_api") == "blas"]
+    if not pools:
+        raise SystemExit("bench.py: cannot tell how many threads numpy's BLAS uses (no BLAS pool reported by threadpoolctl)")
+    threads = max(pools)
     instr = next(i for i in fw.instructions if type(i).__name__ == "AttnInstr")
     mask = np.asarray(instr.attn_mask)
     if mask.ndim == 2:

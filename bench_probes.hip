@@ -1,5 +1,8 @@
-// Two probes for the roofline discussion (no counterpart in the reference; used by bench.py
-// only): the sustained matrix-core rate and the streaming rate of HBM.
+// libbench_probes.so: two measurement-only kernels that bench.py runs beside the product library
+// for the roofline discussion (not part of libdcp_hip.so or of its C ABI; nothing in the
+// reference corresponds to them): the sustained matrix-core rate and the streaming rate of HBM.
+// Built by `python -m dcp_amd.build` from this one file; entry points return 0 or a DCP_ERR_*
+// code and bench_probe_last_error() gives the message.
 //
 // Sustained matrix-core rate of the device: a kernel that does
 // nothing but 32x32x16 MFMAs on operands the caller provides.  What the chip sustains depends
@@ -8,6 +11,12 @@
 #include "attn_common.h"
 
 namespace dcp {
+
+// this library's own message buffer (libdcp_hip.so keeps its own)
+char* last_error_buffer() {
+  static thread_local char buffer[512] = {0};
+  return buffer;
+}
 
 constexpr int kProbeThreads = 256;
 constexpr int kProbeMfmaPerIter = 32;
@@ -81,7 +90,12 @@ __global__ __launch_bounds__(256) void hbm_stream_kernel(const u32x4* __restrict
 
 using namespace dcp;
 
-extern "C" int dcp_hbm_stream_probe(const void* src, void* dst, int n_streams, size_t bytes_per_stream,
+extern "C" const char* bench_probe_last_error(void) { return dcp::last_error_buffer(); }
+
+// Adds `n_streams` (1, 2 or 4) equally long input streams, laid end to end in `src`, 16 bytes at
+// a time and writes the sum to `dst`: n_streams reads and one write of `bytes_per_stream` (a
+// multiple of 8192) each.  Time it with events on `stream`.
+extern "C" int bench_hbm_stream_probe(const void* src, void* dst, int n_streams, size_t bytes_per_stream,
                                     void* stream) {
   DCP_REQUIRE(src && dst, "hbm_stream_probe: null argument");
   DCP_REQUIRE(bytes_per_stream > 0 && bytes_per_stream % (256 * 2 * 16) == 0,
@@ -105,7 +119,12 @@ extern "C" int dcp_hbm_stream_probe(const void* src, void* dst, int n_streams, s
   return check_launch("hbm_stream_kernel");
 }
 
-extern "C" int dcp_mfma_probe(const void* operands, float* out, int n_workgroups, int iters, int dtype,
+// Launches `n_workgroups` workgroups of 256 threads that do nothing but 32x32x16 MFMAs (`iters` x 32
+// per wave) on operands read once from `operands`: 16 x 16 bytes per thread.  `out` receives
+// 2 + n_workgroups * 256 floats: out[0] = shader clocks and out[1] = 100 MHz ticks spent in the
+// loop by workgroup 0, the rest one checksum per thread.  *flop = the floating-point operations
+// the launch performs; time it with events on `stream`.
+extern "C" int bench_mfma_probe(const void* operands, float* out, int n_workgroups, int iters, int dtype,
                               double* flop, void* stream) {
   DCP_REQUIRE(operands && out && flop, "mfma_probe: null argument");
   DCP_REQUIRE(n_workgroups > 0 && iters > 0, "mfma_probe: sizes must be positive");

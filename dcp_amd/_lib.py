@@ -25,8 +25,6 @@ SIGNATURES = {
     "dcp_last_error": [],
     "dcp_profile_enable": [_I],
     "dcp_profile_report": [c_char_p, c_size_t],
-    "dcp_mfma_probe": [_P, _P, _I, _I, _I, _P, _P],
-    "dcp_hbm_stream_probe": [_P, _P, _I, c_size_t, _P],
     "dcp_fused_copy_varlen": [_P, _P, _P, _P, _P, _P, _P, _I, _L, _I, _P],
     "dcp_fused_copy_varlen_dkv": [_P, _P, _P, _I, _I, _I, _I, _P],
     "dcp_fused_copy_varlen_lse": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

@@ -91,7 +91,24 @@ def build_abi_host_check(verbose: bool = True) -> Path:
     return HOST_CHECK_BIN
 
 
+PROBES_SRC = PKG_DIR.parent / "bench_probes.hip"
+PROBES_LIB = PKG_DIR.parent / "libbench_probes.so"
+
+
+def build_bench_probes(verbose: bool = True) -> Path:
+    """Compiles bench_probes.hip (two measurement-only kernels that bench.py runs beside the
+    product library) into libbench_probes.so next to bench.py.  Not part of libdcp_hip.so."""
+    cmd = [HIPCC, *FLAGS, "-shared", str(PROBES_SRC), "-o", str(PROBES_LIB)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"bench probes failed to build:\n{proc.stderr}")
+    if verbose:
+        print(f"built {PROBES_LIB}", file=sys.stderr)
+    return PROBES_LIB
+
+
 if __name__ == "__main__":
     build()
     if LIB_PATH.name == "libdcp_hip.so":  # the host check links the library by its name
         build_abi_host_check()
+        build_bench_probes()

@@ -25,18 +25,25 @@ std::vector<Span> g_spans;
 
 bool profiling_enabled() { return g_profiling; }
 
-void profile_begin(const char* name, hipStream_t stream) {
+int profile_begin(const char* name, hipStream_t stream) {
   std::lock_guard<std::mutex> lock(g_mu);
   Span s;
   s.name = name;
-  if (hipEventCreate(&s.start) != hipSuccess || hipEventCreate(&s.stop) != hipSuccess) return;
+  if (hipEventCreate(&s.start) != hipSuccess) return -1;
+  if (hipEventCreate(&s.stop) != hipSuccess) {
+    (void)hipEventDestroy(s.start);
+    return -1;
+  }
   (void)hipEventRecord(s.start, stream);
   g_spans.push_back(s);
+  return (int)g_spans.size() - 1;
 }
 
-void profile_end(hipStream_t stream) {
+void profile_end(int span, hipStream_t stream) {
   std::lock_guard<std::mutex> lock(g_mu);
-  if (!g_spans.empty()) (void)hipEventRecord(g_spans.back().stop, stream);
+  // the span this timer opened (none if its events could not be created, or if a report has
+  // cleared the list in between)
+  if (span >= 0 && span < (int)g_spans.size()) (void)hipEventRecord(g_spans[span].stop, stream);
 }
 
 }  // namespace dcp

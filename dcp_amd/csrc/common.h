@@ -52,17 +52,17 @@ inline int device_cu_count() {
 // them and sums the elapsed time per kernel name.  Nothing is recorded, created
 // or synchronised when profiling is off.
 bool profiling_enabled();
-void profile_begin(const char* name, hipStream_t stream);
-void profile_end(hipStream_t stream);
+int profile_begin(const char* name, hipStream_t stream);  // the span's index, or -1 if no events could be made
+void profile_end(int span, hipStream_t stream);
 
 struct KernelTimer {
   hipStream_t stream;
-  bool on;
-  KernelTimer(const char* name, void* s) : stream((hipStream_t)s), on(profiling_enabled()) {
-    if (on) profile_begin(name, stream);
+  int span;
+  KernelTimer(const char* name, void* s) : stream((hipStream_t)s), span(-1) {
+    if (profiling_enabled()) span = profile_begin(name, stream);
   }
   ~KernelTimer() {
-    if (on) profile_end(stream);
+    if (span >= 0) profile_end(span, stream);
   }
 };
 

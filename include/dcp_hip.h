@@ -54,31 +54,6 @@ void dcp_profile_enable(int on);
 int dcp_profile_report(char* buffer, size_t capacity);
 
 /*
- * Sustained matrix-core rate of the device, for the roofline discussion (no
- * counterpart in the reference; used by the benchmark only).  Launches
- * `n_workgroups` workgroups of 256 threads that do nothing but 32x32x16 MFMAs
- * (`iters` x 32 per wave) on operands read once from `operands`: 16 x 16 bytes
- * per thread, n_workgroups * 256 * 256 bytes in all; what the chip sustains
- * depends on their values (constant operands run at the full shader clock,
- * random ones do not).  `out` receives 2 + n_workgroups * 256 floats: out[0] =
- * shader clocks and out[1] = 100 MHz ticks spent in the loop by workgroup 0, the
- * rest one checksum per thread.  *flop = the floating-point operations the
- * launch performs; time it with events on `stream`.
- */
-int dcp_mfma_probe(const void* operands, float* out, int n_workgroups, int iters, int dtype,
-                   double* flop, void* stream);
-
-/*
- * Streaming rate of HBM, for the roofline discussion (no counterpart in the
- * reference; used by the benchmark only).  Adds `n_streams` (1, 2 or 4) equally
- * long input streams, laid end to end in `src`, 16 bytes at a time and writes
- * the sum to `dst`: n_streams reads and one write of `bytes_per_stream` (a
- * multiple of 8192) each.  Time it with events on `stream`.
- */
-int dcp_hbm_stream_probe(const void* src, void* dst, int n_streams, size_t bytes_per_stream,
-                         void* stream);
-
-/*
  * Block gather / scatter through pointer tables.
  * Replaces dcp.ops.fused_ops.fused_copy_{bf16,fp16,fp32}_varlen
  * (dcp/ops/fused_ops.py:842-864, 916-938, 1013-1035; kernels :290-335,

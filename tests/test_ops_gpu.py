@@ -319,12 +319,12 @@ def test_fused_blockwise_sum_rejects_dtype(gpu):
 
 
 def test_roofline_probes(gpu):
-    """The two measurement-only entry points: the streaming probe's output is the exact
-    (wrap-around) 32-bit sum of its streams, the MFMA probe reports its FLOP count and clocks,
-    and both reject what they do not support."""
+    """The benchmark's two measurement-only kernels (bench_probes.hip, a library of their own):
+    the streaming probe's output is the exact (wrap-around) 32-bit sum of its streams, the MFMA
+    probe reports its FLOP count and clocks, and both reject what they do not support."""
     import ctypes
 
-    from dcp_amd import _lib
+    from bench import call_probe
 
     stream = torch.cuda.current_stream().cuda_stream
     per_stream = 8192 * 64
@@ -332,24 +332,24 @@ def test_roofline_probes(gpu):
     src = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=4 * per_stream // 4, dtype=np.int64).astype(np.int32)).to(gpu)
     dst = torch.zeros(per_stream // 4, dtype=torch.int32, device=gpu)
     for n in (1, 2, 4):
-        _lib.call("dcp_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), n, per_stream, stream)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), n, per_stream, stream)
         torch.cuda.synchronize()
         want = src.reshape(4, -1)[:n].to(torch.int64).sum(0).to(torch.int32)  # wraps like the 32-bit adds
         assert torch.equal(dst, want), n
     with pytest.raises(ValueError):
-        _lib.call("dcp_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 3, per_stream, stream)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 3, per_stream, stream)
     with pytest.raises(AssertionError):
-        _lib.call("dcp_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 1, 100, stream)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 1, 100, stream)
 
     n_wg, iters = 8, 10
     ops = torch.full((n_wg * 256 * 16 * 8,), 0.5, device=gpu, dtype=torch.bfloat16)
     out = torch.zeros(2 + n_wg * 256, device=gpu)
     flop = ctypes.c_double()
-    _lib.call("dcp_mfma_probe", ops.data_ptr(), out.data_ptr(), n_wg, iters, 0, ctypes.byref(flop), stream)
+    call_probe("bench_mfma_probe", ops.data_ptr(), out.data_ptr(), n_wg, iters, 0, ctypes.byref(flop), stream)
     torch.cuda.synchronize()
     assert flop.value == n_wg * 4 * iters * 32 * 2.0 * 32 * 32 * 16
     assert out[0].item() > 0 and out[1].item() > 0
     # every accumulator element of the probe is iters * 32 / 4 products of 16 terms 0.5 * 0.5
     assert torch.allclose(out[2:], torch.full_like(out[2:], 64 * (iters * 32 / 4) * 16 * 0.25))
     with pytest.raises(ValueError):
-        _lib.call("dcp_mfma_probe", ops.data_ptr(), out.data_ptr(), n_wg, iters, 2, ctypes.byref(flop), stream)
+        call_probe("bench_mfma_probe", ops.data_ptr(), out.data_ptr(), n_wg, iters, 2, ctypes.byref(flop), stream)
