@@ -56,7 +56,10 @@ __device__ __forceinline__ bool lse_is_finite(float l) {
 // transaction), so no cross-lane traffic is needed.  Because the group sits
 // inside one wave and each lane only overwrites elements it has already read,
 // the destination may alias a source of the same op.
-// grid: (ops, token chunks x heads)
+// grid: ops x (token chunks x heads), one dimension with the chunks of an op side by side:
+// workgroups that run at the same time then read neighbouring pieces of the same few blocks
+// (with the op as the fastest index, as a two-dimensional grid has it, they are spread over
+// all the blocks of the launch at once).
 // ---------------------------------------------------------------------------
 constexpr int kMergeThreads = 256;
 
@@ -70,18 +73,19 @@ __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
     const int32_t* __restrict__ dst_token_offsets, const int32_t* __restrict__ n_tokens_per_block,
     const int32_t* __restrict__ block_lengths, int64_t out_block_stride, int64_t out_token_stride,
     int64_t lse_block_stride, int64_t lse_token_stride, int64_t src_lse_head_stride,
-    int64_t dst_lse_head_stride, int head_dim, int max_n_blocks_per_op, int lanes_per_row) {
+    int64_t dst_lse_head_stride, int head_dim, int max_n_blocks_per_op, int lanes_per_row, int row_chunks) {
   typedef typename Elem<DTYPE>::raw raw;
   constexpr int VN = VECTOR ? Vec16<DTYPE>::N : 1;
-  const int op = blockIdx.x;
+  const int op = blockIdx.x / row_chunks;
+  const int chunk = blockIdx.x - op * row_chunks;
   const int n_tok = n_tokens_per_block[op];
 
   // A workgroup takes consecutive tokens of ONE head: its LSE reads and its LSE store are
   // then contiguous floats ([head][token] layout) instead of one 4-byte access per cache
   // line, and every token's head_dim elements are still one contiguous piece.
   const int rows_per_wg = kMergeThreads / lanes_per_row;
-  const int h = blockIdx.y % n_head;
-  const int t0 = (blockIdx.y / n_head) * (rows_per_wg * TPG) + threadIdx.x / lanes_per_row;
+  const int h = chunk % n_head;
+  const int t0 = (chunk / n_head) * (rows_per_wg * TPG) + threadIdx.x / lanes_per_row;
   const int g = threadIdx.x % lanes_per_row;
   if (t0 >= n_tok) return;
 
@@ -202,6 +206,132 @@ __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same merge for the layout plans have: token rows that are dense over the heads
+// (out_token_stride = n_head * head_dim) and LSEs contiguous over tokens.  A workgroup takes
+// kRowTokens consecutive tokens of one op with ALL their heads, so that every global access of
+// the out data is part of a run of whole token rows (4 KiB per wave instruction at 32 heads x
+// 128 bf16) instead of one 256-byte piece per 8 KiB, and works in two phases:
+//   A  the sources' LSEs of its (head, token) pairs -> the merged LSE (stored) and one weight
+//      exp(l_j - lse*) per (source, head, token), kept in LDS (0 for an ignored source);
+//   B  out* = sum_j w_j out_j, 16 bytes per lane and source, kRowUnroll words in flight.
+// grid: ops x token chunks, an op's chunks side by side
+// ---------------------------------------------------------------------------
+constexpr int kRowTokens = 2;   // measured on 262144 tokens x 32 heads x 128 bf16, four sources: 16 tokens per
+constexpr int kRowUnroll = 2;   // workgroup 5.36 TB/s, 4: 5.53, 2: 5.98, 1: 5.69; four words per source in flight: 5.53
+constexpr int kRowWeightFloats = 12288;  // LDS for the weights: n_src * n_head * kRowTokens floats at most
+
+template <int DTYPE, int U>
+__global__ __launch_bounds__(kMergeThreads) void merge_rows_kernel(
+    const typename Elem<DTYPE>::raw* src_out, typename Elem<DTYPE>::raw* dst_out, const float* src_lse,
+    float* dst_lse, int n_head, const int32_t* __restrict__ src_block_table,
+    const int32_t* __restrict__ dst_token_offsets, const int32_t* __restrict__ n_tokens_per_block,
+    const int32_t* __restrict__ block_lengths, int64_t out_block_stride, int64_t out_token_stride,
+    int64_t lse_block_stride, int64_t src_lse_head_stride, int64_t dst_lse_head_stride, int head_dim,
+    int max_n_blocks_per_op, int chunks_per_op) {
+  typedef typename Elem<DTYPE>::raw raw;
+  constexpr int VN = Vec16<DTYPE>::N;
+  extern __shared__ float weight[];  // [source][head][token of the chunk]: max_n_blocks_per_op * n_head * kRowTokens
+  const int op = blockIdx.x / chunks_per_op;
+  const int n_tok = n_tokens_per_block[op];
+  const int t0 = (blockIdx.x - op * chunks_per_op) * kRowTokens;
+  if (t0 >= n_tok) return;
+  const int n_src = block_lengths[op];
+  const int tid = threadIdx.x;
+  const int32_t* slot = src_block_table + (int64_t)op * max_n_blocks_per_op;  // the same for the whole workgroup: scalar loads
+  const int64_t dst_tok0 = (int64_t)dst_token_offsets[op] + t0;
+  const int plane = n_head * kRowTokens;
+  const int words_per_head = head_dim / VN;
+  const int row_words = n_head * words_per_head;
+  const int n_rows = min(kRowTokens, n_tok - t0);
+  const int total = n_rows * row_words;
+
+  // word i of the chunk: token i / row_words, 16-byte word i % row_words of its row
+  auto load_words = [&](u32x4 (&x)[U][kRowUnroll], const int (&t)[kRowUnroll], const int (&wd)[kRowUnroll], int j0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int j = min(j0 + u, n_src - 1);  // tail: re-read the last source, ignored by the caller
+      const raw* base = src_out + (int64_t)slot[j] * out_block_stride + (int64_t)t0 * out_token_stride;
+#pragma unroll
+      for (int k = 0; k < kRowUnroll; ++k)
+        x[u][k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + (int64_t)t[k] * out_token_stride + (int64_t)wd[k] * VN));
+    }
+  };
+  auto locate = [&](int i0, int (&t)[kRowUnroll], int (&wd)[kRowUnroll], bool (&live)[kRowUnroll]) {
+#pragma unroll
+    for (int k = 0; k < kRowUnroll; ++k) {
+      const int i = i0 + k * kMergeThreads;
+      live[k] = i < total;
+      const int ii = live[k] ? i : i0;
+      t[k] = ii / row_words;
+      wd[k] = ii - t[k] * row_words;
+    }
+  };
+
+  // ---- phase A --------------------------------------------------------------------------
+  for (int pair = tid; pair < plane; pair += kMergeThreads) {
+    const int h = pair / kRowTokens, t = pair - h * kRowTokens;
+    if (t0 + t >= n_tok) continue;
+    const float* lse_row = src_lse + (int64_t)h * src_lse_head_stride + t0 + t;
+    float m = -INFINITY;
+    for (int j = 0; j < n_src; ++j) {
+      float l = lse_row[(int64_t)slot[j] * lse_block_stride];
+      if (!lse_is_finite(l)) l = -INFINITY;
+      weight[j * plane + pair] = l;
+      m = fmaxf(m, l);
+    }
+    float new_lse = -1.0f;
+    if (m != -INFINITY) {
+      float ssum = 0.0f;
+      for (int j = 0; j < n_src; ++j) ssum += expf(weight[j * plane + pair] - m);  // ignored source: exp(-inf) = 0
+      new_lse = m + logf(ssum);
+      // a single source keeps its LSE bit for bit (m + log(1) may round)
+      if (n_src == 1) new_lse = weight[pair];
+    }
+    for (int j = 0; j < n_src; ++j) {
+      const float l = weight[j * plane + pair];
+      weight[j * plane + pair] = (m == -INFINITY || l == -INFINITY) ? 0.0f : expf(l - new_lse);
+    }
+    // (after this pair's reads: the destination may be one of its sources)
+    dst_lse[(int64_t)h * dst_lse_head_stride + dst_tok0 + t] = new_lse;
+  }
+  __syncthreads();
+
+  // ---- phase B --------------------------------------------------------------------------
+  const bool copy_only = n_src == 1;  // the scatter-back of a finished block: bits, not 0 + 1 * x
+  for (int i0 = tid; i0 < total; i0 += kMergeThreads * kRowUnroll) {
+    int t[kRowUnroll], wd[kRowUnroll];
+    bool live[kRowUnroll];
+    float acc[kRowUnroll][VN];
+    locate(i0, t, wd, live);
+#pragma unroll
+    for (int k = 0; k < kRowUnroll; ++k)
+#pragma unroll
+      for (int e = 0; e < VN; ++e) acc[k][e] = 0.0f;
+    u32x4 only[kRowUnroll];
+    for (int j0 = 0; j0 < n_src; j0 += U) {
+      u32x4 x[U][kRowUnroll];
+      load_words(x, t, wd, j0);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (j0 + u >= n_src) break;
+#pragma unroll
+        for (int k = 0; k < kRowUnroll; ++k) {
+          const float w = weight[(j0 + u) * plane + (wd[k] / words_per_head) * kRowTokens + t[k]];
+          if (w != 0.0f) fma_vec16<DTYPE>(acc[k], w, x[u][k]);  // an ignored source's data may be anything: skipped
+          if (u == 0) only[k] = w != 0.0f ? x[0][k] : u32x4{0, 0, 0, 0};
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kRowUnroll; ++k) {
+      if (!live[k]) continue;
+      raw* q = dst_out + (dst_tok0 + t[k]) * out_token_stride + (int64_t)wd[k] * VN;
+      __builtin_nontemporal_store(copy_only ? only[k] : pack_vec16<DTYPE>(acc[k]), reinterpret_cast<u32x4*>(q));
+    }
+  }
+}
+
 template <int DTYPE>
 static int launch_merge(const void* src_out, void* dst_out, const float* src_lse, float* dst_lse,
                         int n_head, const int32_t* src_block_table,
@@ -217,6 +347,25 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
                    out_token_stride % VN == 0 &&
                    ((reinterpret_cast<uintptr_t>(src_out) | reinterpret_cast<uintptr_t>(dst_out)) &
                     15) == 0;
+  // the row-streaming kernel, when rows are dense over the heads and the weights fit in LDS
+  if (vec && out_token_stride == (int64_t)n_head * head_dim && lse_token_stride == 1 &&
+      (int64_t)max_n_blocks_per_op * n_head * kRowTokens <= kRowWeightFloats) {
+    const int64_t chunks = (block_size + kRowTokens - 1) / kRowTokens;
+    DCP_REQUIRE(chunks * n_red_ops < ((int64_t)1 << 31), "merge: too many (op, token chunk) items");
+    dim3 grid((unsigned)(chunks * n_red_ops));
+    KernelTimer timer("merge_out_lse_kernel", stream);
+    auto launch_rows = [&](auto kernel) {
+      const size_t lds_bytes = (size_t)max_n_blocks_per_op * n_head * kRowTokens * sizeof(float);
+      hipLaunchKernelGGL(kernel, grid, dim3(kMergeThreads), lds_bytes, (hipStream_t)stream, (const raw*)src_out, (raw*)dst_out,
+                         src_lse, dst_lse, n_head, src_block_table, dst_token_offsets, n_tokens_per_block, block_lengths,
+                         out_block_stride, out_token_stride, lse_block_stride, src_lse_head_stride, dst_lse_head_stride,
+                         head_dim, max_n_blocks_per_op, (int)chunks);
+    };
+    if (max_n_blocks_per_op >= 4) launch_rows(merge_rows_kernel<DTYPE, 4>);
+    else if (max_n_blocks_per_op >= 2) launch_rows(merge_rows_kernel<DTYPE, 2>);
+    else launch_rows(merge_rows_kernel<DTYPE, 1>);
+    return check_launch("merge_out_lse_kernel");
+  }
   const int n_words = vec ? head_dim / VN : head_dim;
   int lpr = 1;
   while (lpr < 64 && n_words % (lpr * 2) == 0) lpr *= 2;
@@ -226,16 +375,16 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
   const int u = max_n_blocks_per_op >= 4 ? 4 : max_n_blocks_per_op >= 2 ? 2 : 1;
   const int tpg = u == 4 ? 2 : u == 2 ? 4 : 2;
   const int64_t row_chunks = (int64_t)((block_size + rows_per_wg * tpg - 1) / (rows_per_wg * tpg)) * n_head;
-  DCP_REQUIRE(row_chunks <= 65535, "merge: block of %lld (token, head) rows is too large",
-              (long long)block_size * n_head);
-  dim3 grid(n_red_ops, (unsigned)row_chunks);
+  DCP_REQUIRE(row_chunks * n_red_ops < ((int64_t)1 << 31), "merge: %d ops of %lld (token, head) rows are too many for one launch",
+              n_red_ops, (long long)block_size * n_head);
+  dim3 grid((unsigned)(row_chunks * n_red_ops));
   KernelTimer timer("merge_out_lse_kernel", stream);
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(kMergeThreads), 0, (hipStream_t)stream, (const raw*)src_out,
                        (raw*)dst_out, src_lse, dst_lse, n_head, src_block_table,
                        dst_token_offsets, n_tokens_per_block, block_lengths, out_block_stride,
                        out_token_stride, lse_block_stride, lse_token_stride, src_lse_head_stride,
-                       dst_lse_head_stride, head_dim, max_n_blocks_per_op, lpr);
+                       dst_lse_head_stride, head_dim, max_n_blocks_per_op, lpr, (int)row_chunks);
   };
 #define DCP_MERGE_PICK(V)                                           \
   do {                                                              \
@@ -250,7 +399,7 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
 }
 
 // ---------------------------------------------------------------------------
-// Block sum.  grid: (sums, chunks of 256*16 bytes*UNROLL)
+// Block sum.  grid: sums x chunks of 256*16 bytes*UNROLL, one dimension with a sum's chunks side by side
 // ---------------------------------------------------------------------------
 constexpr int kSumUnroll = 2;
 
@@ -260,13 +409,13 @@ __global__ __launch_bounds__(256) void blockwise_sum_kernel(
     const int32_t* __restrict__ src_strides, const int32_t* __restrict__ n_ops_per_block,
     const int64_t* __restrict__ dst_ptrs, const int32_t* __restrict__ dst_offsets,
     const int32_t* __restrict__ dst_strides, const int32_t* __restrict__ n_elements,
-    int max_n_ops_per_block) {
+    int max_n_ops_per_block, int chunks_per_sum) {
   typedef typename Elem<DTYPE>::raw raw;
   constexpr int VN = Vec16<DTYPE>::N;
-  const int s = blockIdx.x;
+  const int s = blockIdx.x / chunks_per_sum;
   const int64_t n_elem = n_elements[s];
   const int64_t chunk_elems = (int64_t)256 * VN * kSumUnroll;
-  const int64_t begin = (int64_t)blockIdx.y * chunk_elems;
+  const int64_t begin = (int64_t)(blockIdx.x - s * chunks_per_sum) * chunk_elems;
   if (begin >= n_elem) return;
   const int64_t end = min(begin + chunk_elems, n_elem);
 
@@ -391,13 +540,14 @@ extern "C" int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_off
               "sum: null table");
   const int64_t chunk_elems = (int64_t)256 * (16 / esize) * kSumUnroll;
   const int64_t chunks = (block_numel + chunk_elems - 1) / chunk_elems;
-  DCP_REQUIRE(chunks <= 65535, "sum: block of %lld elements is too large", (long long)block_numel);
-  dim3 grid(n_sums, (unsigned)chunks);
+  DCP_REQUIRE(chunks * n_sums < ((int64_t)1 << 31), "sum: %d sums of %lld elements are too many for one launch", n_sums,
+              (long long)block_numel);
+  dim3 grid((unsigned)(chunks * n_sums));
   KernelTimer timer("blockwise_sum_kernel", stream);
 #define DCP_SUM_LAUNCH(DT)                                                                     \
   hipLaunchKernelGGL(blockwise_sum_kernel<DT>, grid, dim3(256), 0, (hipStream_t)stream,        \
                      src_ptrs, src_offsets, src_strides, n_ops_per_block, dst_ptrs,            \
-                     dst_offsets, dst_strides, n_elements, max_n_ops_per_block)
+                     dst_offsets, dst_strides, n_elements, max_n_ops_per_block, (int)chunks)
   switch (dtype) {
     case DCP_DTYPE_BF16:
       DCP_SUM_LAUNCH(DCP_DTYPE_BF16);
