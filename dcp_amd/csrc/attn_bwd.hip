@@ -1,16 +1,19 @@
 // Range-masked paged attention backward for gfx950.
 //
-// Two small kernels and two big ones per call:
+// One small kernel and two big ones per call, in this order:
 //
-//   bwd_prep_kernel      delta[q, h] = -sum_d dO*O  (negated: it is added, as an accumulator's initial value)
 //   bwd_tile_hull_kernel per (row, 64-query tile): hull and core of the rows'
 //                        key ranges, so the dK/dV kernel can skip / unmask tiles
+//   attn_bwd_dq_kernel   query-outer: one workgroup per (row, head, 128-query
+//                        tile) walks the key tiles and keeps dQ^T in registers.
+//                        Its prologue also computes -delta[q, h] = -sum_d dO*O
+//                        (negated: it is added, as an accumulator's initial
+//                        value) and the base-2 log-sum-exp of its queries and
+//                        leaves them in the workspace for the next kernel
 //   attn_bwd_dkv_kernel  key-outer: one workgroup per (row, 128-key tile, kv
 //                        head) loops over the q heads of the kv head's group
 //                        and the 64-query tiles of the row and keeps dK^T and
 //                        dV^T of its keys in registers
-//   attn_bwd_dq_kernel   query-outer: one workgroup per (row, head, 128-query
-//                        tile) walks the key tiles and keeps dQ^T in registers
 //
 // dQ and dK/dV each get the loop order that keeps them in registers; S and dP
 // are recomputed in the second kernel (7 matrix products instead of 5).  The
@@ -63,7 +66,7 @@ struct AttnBwdParams {
   void* dk;
   void* dv;
   float* delta;      // [total_q, H]: MINUS rowsum(dO * O)
-  float* lse2;       // [total_q, H]: lse * log2(e), written by the prep kernel for the dK/dV kernel
+  float* lse2;       // [total_q, H]: lse * log2(e); both written by the dQ kernel, read by the dK/dV kernel
   int32_t* hull;     // [batch * q_tiles_per_row, 8]
   int* tickets;      // work-item counters of the persistent dQ kernel (kTicketInts); zeroed by the hull kernel
   const int32_t* cu_seqlens_q;
@@ -102,42 +105,6 @@ constexpr int kBwdBM = 64;
 constexpr int kBwdBN = 64;
 constexpr int kBwdThreads = 256;
 constexpr int kTicketInts = 16;  // one counter per XCD (the rest unused)
-
-// ---------------------------------------------------------------------------
-// delta[q, h] = -sum_d dO*O.  LPR lanes per (token, head) row, 8 elements each.
-// grid: (batch, row chunks)
-// ---------------------------------------------------------------------------
-template <int DTYPE, int D>
-__global__ __launch_bounds__(256) void bwd_prep_kernel(const AttnBwdParams p) {
-  constexpr int LPR = D / 8;
-  constexpr int ROWS = 256 / LPR;
-  const int b = blockIdx.x;
-  const int q_begin = p.cu_seqlens_q[b];
-  const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
-  const int row = blockIdx.y * ROWS + threadIdx.x / LPR;
-  const int g = threadIdx.x % LPR;
-  const int t = row / p.n_heads_q;
-  const int hd = row - t * p.n_heads_q;
-  if (t >= seqlen_q) return;  // whole LPR-lane group leaves together
-  const int64_t off = (((int64_t)p.out_block_table[b] * p.block_size + t) * p.n_heads_q + hd) * D + g * 8;
-  const u32x4 o = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.out) + off);
-  const u32x4 d = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.dout) + off);
-  float acc = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    acc += Elem<DTYPE>::load((uint16_t)(o[i] & 0xffffu)) * Elem<DTYPE>::load((uint16_t)(d[i] & 0xffffu));
-    acc += Elem<DTYPE>::load((uint16_t)(o[i] >> 16)) * Elem<DTYPE>::load((uint16_t)(d[i] >> 16));
-  }
-#pragma unroll
-  for (int o2 = LPR / 2; o2 > 0; o2 >>= 1) acc += __shfl_xor(acc, o2);
-  const int64_t qrow = ((int64_t)(q_begin + t) * p.n_heads_q + hd);
-  if (g == 0) {
-    p.delta[qrow] = -acc;
-    // the log-sum-exp in the base-2 domain the kernels work in, one multiply per (token, head)
-    // here instead of one per (query, key tile) in the dK/dV kernel's vector phase
-    p.lse2[qrow] = p.lse[((int64_t)hd * p.n_out_slots + p.out_block_table[b]) * p.block_size + t] * kLog2e;
-  }
-}
 
 // One wave per (row, 64-query tile).  hull[0..3] = lo0, hi0, lo1, hi1 over
 // rows with a non-empty range; hull[4..7] = the intersection (core) of the
@@ -556,24 +523,41 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
   const bool q_valid = q_local < seqlen_q;
   const int o_slot = p.out_block_table[b];
 
-  // Q and dO fragments of this lane's query row (B operands), lse and delta
+  // Q and dO fragments of this lane's query row (B operands), and the row's two scalars: the
+  // base-2 log-sum-exp and -delta = -sum_d dO * O.  The lane holds half of the row's dims (those
+  // of its k-slots), so delta is the lane's partial dot product plus the other half-wave's.  Both
+  // scalars are also stored for the dK/dV kernel, which runs after this one and reads them per
+  // (query, head) from the workspace: every (row, head, valid query) is written exactly once.
   u32x4 qreg[KS], doreg[KS];
   float lse2 = INFINITY, delta = 0.0f;
   {
     const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) +
                          ((int64_t)p.q_block_table[b] * p.block_size + q_local) * q_row_stride +
                          (int64_t)head * D + h * 8;
-    const uint16_t* dp = reinterpret_cast<const uint16_t*>(p.dout) +
-                         ((int64_t)o_slot * p.block_size + q_local) * q_row_stride + (int64_t)head * D + h * 8;
+    const int64_t o_off = ((int64_t)o_slot * p.block_size + q_local) * q_row_stride + (int64_t)head * D + h * 8;
+    const uint16_t* dp = reinterpret_cast<const uint16_t*>(p.dout) + o_off;
+    const uint16_t* op = reinterpret_cast<const uint16_t*>(p.out) + o_off;
+    float dot = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 z = {0, 0, 0, 0};
       qreg[ks] = q_valid ? *reinterpret_cast<const u32x4*>(qp + ks * 16) : z;
       doreg[ks] = q_valid ? *reinterpret_cast<const u32x4*>(dp + ks * 16) : z;
+      const u32x4 o = q_valid ? *reinterpret_cast<const u32x4*>(op + ks * 16) : z;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        dot += Elem<DTYPE>::load((uint16_t)(o[i] & 0xffffu)) * Elem<DTYPE>::load((uint16_t)(doreg[ks][i] & 0xffffu));
+        dot += Elem<DTYPE>::load((uint16_t)(o[i] >> 16)) * Elem<DTYPE>::load((uint16_t)(doreg[ks][i] >> 16));
+      }
     }
+    delta = -halves_sum(dot);
     if (q_valid) {
       lse2 = p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local] * kLog2e;
-      delta = p.delta[(int64_t)(q_begin + q_local) * p.n_heads_q + head];
+      if (h == 0) {
+        const int64_t qrow = (int64_t)(q_begin + q_local) * p.n_heads_q + head;
+        p.delta[qrow] = delta;
+        p.lse2[qrow] = lse2;
+      }
     }
   }
   RangePair rng = {0, 0, 0, 0};
@@ -797,29 +781,21 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_kernel(const AttnB
 
 template <int DTYPE, int D>
 static int launch_bwd(const AttnBwdParams& p, hipStream_t stream) {
-  constexpr int ROWS = 256 / (D / 8);
-  const int64_t rows = (int64_t)p.block_size * p.n_heads_q;
-  const int64_t chunks = (rows + ROWS - 1) / ROWS;
-  DCP_REQUIRE(chunks <= 65535, "attn_bwd: block of %lld (token, head) rows is too large", (long long)rows);
   const int64_t n_dkv = xcd_grid_size(p.n_dkv_items, p.dkv_xcd_group);
   DCP_REQUIRE(n_dkv < ((int64_t)1 << 31) && p.n_dq_items < ((int64_t)1 << 31), "attn_bwd: grid too large");
   // as many workgroups as the device holds at once (two per CU), a multiple of the XCD count
   const int64_t n_dq = std::min<int64_t>(xcd_grid_size(p.n_dq_items, 1), xcd_grid_size(2 * (int64_t)device_cu_count(), 1));
   {
-    KernelTimer timer("bwd_prep_kernel", stream);
-    hipLaunchKernelGGL((bwd_prep_kernel<DTYPE, D>), dim3(p.batch, (unsigned)chunks), dim3(256), 0, stream, p);
-  }
-  {
     KernelTimer timer("bwd_tile_hull_kernel", stream);
     hipLaunchKernelGGL(bwd_tile_hull_kernel, dim3(p.batch * p.q_tiles_per_row), dim3(64), 0, stream, p);
+  }
+  {  // first: it also leaves -delta and the base-2 LSE of every query in the workspace for the dK/dV kernel
+    KernelTimer timer("attn_bwd_dq_kernel", stream);
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<DTYPE, D>), dim3((unsigned)n_dq), dim3(kBwdThreads), 0, stream, p);
   }
   {
     KernelTimer timer("attn_bwd_dkv_kernel", stream);
     hipLaunchKernelGGL((attn_bwd_dkv_kernel<DTYPE, D>), dim3((unsigned)n_dkv), dim3(kBwdThreads), 0, stream, p);
-  }
-  {
-    KernelTimer timer("attn_bwd_dq_kernel", stream);
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<DTYPE, D>), dim3((unsigned)n_dq), dim3(kBwdThreads), 0, stream, p);
   }
   return check_launch("attn_bwd kernels");
 }

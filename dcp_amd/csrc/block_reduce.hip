@@ -347,8 +347,11 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
                    out_token_stride % VN == 0 &&
                    ((reinterpret_cast<uintptr_t>(src_out) | reinterpret_cast<uintptr_t>(dst_out)) &
                     15) == 0;
-  // the row-streaming kernel, when rows are dense over the heads and the weights fit in LDS
+  // the row-streaming kernel, when rows are dense over the heads, wide enough to give every lane of
+  // its workgroups work (a head block of 4 x 128 bf16 is not: 0.48 ms against 0.20 for the
+  // single-source merge of the 65536-token benchmark step) and the weights fit in LDS
   if (vec && out_token_stride == (int64_t)n_head * head_dim && lse_token_stride == 1 &&
+      (int64_t)n_head * head_dim / VN * kRowTokens >= kMergeThreads * kRowUnroll &&
       (int64_t)max_n_blocks_per_op * n_head * kRowTokens <= kRowWeightFloats) {
     const int64_t chunks = (block_size + kRowTokens - 1) / kRowTokens;
     DCP_REQUIRE(chunks * n_red_ops < ((int64_t)1 << 31), "merge: too many (op, token chunk) items");

@@ -196,6 +196,19 @@ def test_update_out_lse_in_place_fold(gpu):
     assert err_out <= 2e-2 and err_lse <= 1e-3
 
 
+@pytest.mark.parametrize("name,tol", [("fp32", 2e-5), ("bf16", 2e-2), ("fp16", 4e-3)])
+def test_update_out_lse_wide_rows(gpu, name, tol):
+    """Token rows of 4 KiB and more (16 heads x 128, the executor's layout with large head blocks)
+    take the row-streaming kernel: ragged token counts, ignored sources, 1 to 9 sources per op,
+    unpadded destination and the in-place fold."""
+    dtype = DTYPES[name]
+    heads = 16 if name != "fp32" else 8
+    err_out, err_lse = _merge_case(gpu, dtype, [2, 4, 1, 9, 3], heads, 128, 64, seed=5, inf_frac=0.3)
+    assert err_out <= tol and err_lse <= 1e-3, (err_out, err_lse)
+    err_out, err_lse = _merge_case(gpu, dtype, [2, 2, 3], heads, 128, 128, seed=6, unpadded=False)
+    assert err_out <= tol and err_lse <= 1e-3, (err_out, err_lse)
+
+
 def test_update_out_lse_single_source_is_exact_copy(gpu):
     # one finite source: weight exp(l - l) = 1, so the merge is the scatter-back
     err_out, err_lse = _merge_case(gpu, torch.bfloat16, [1, 1, 1, 1], 4, 128, 512, seed=3)
@@ -204,7 +217,8 @@ def test_update_out_lse_single_source_is_exact_copy(gpu):
 
 @pytest.mark.parametrize("name", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("width", [1, 4])
-def test_single_source_merge_and_sum_copy_bit_patterns(gpu, name, width):
+@pytest.mark.parametrize("heads,d", [(3, 64), (16, 128)])  # narrow rows / rows wide enough for the row-streaming merge
+def test_single_source_merge_and_sum_copy_bit_patterns(gpu, name, width, heads, d):
     """Ops with one source are the scatter-back of finished blocks: bit for bit the source,
     negative zeros and NaN payloads included (compared as integers, not as floats), also when
     the launch's table is wide enough for more sources; a source whose LSE is infinite gives
@@ -214,7 +228,7 @@ def test_single_source_merge_and_sum_copy_bit_patterns(gpu, name, width):
     dtype = DTYPES[name]
     ibits = torch.int32 if dtype == torch.float32 else torch.int16
     g = torch.Generator().manual_seed(9)
-    bs, heads, d, n_blocks = 128, 3, 64, 5
+    bs, n_blocks = 128, 5
     src = torch.randn(n_blocks, bs, heads, d, generator=g).to(dtype)
     flat = src.view(ibits).reshape(-1)
     sign = torch.tensor(-0.0, dtype=dtype).view(ibits)  # the sign bit alone = -0.0
