@@ -413,9 +413,17 @@ def build_staged_multi_device_plans(
     stage 0 holds what needs no transfer, the blocks of stage k+1 travel (key ``S{k+1}``) while
     stage k is computed, and a remote block wanted by several devices of a node is received by
     one of them and forwarded inside the node on the second-phase stream (key ``S{k+1}P2``), in
-    the instruction order of ``dcp/core/scheduler.py:894-1049``.  Every (row, stage) writes its
-    own partial; partials meet at the owner of their block through the output exchange ``O``.
-    Slots are never reused.  Returns ``(fw_plans, bw_plans, layouts)`` as the unstaged builder."""
+    the instruction order of ``dcp/core/scheduler.py:894-1049``.  A stage's partial of a block that
+    already has one on the device is folded into the older one right after the stage (merge for
+    out / LSE, sum for dQ; a kv block's private dK/dV replicas are summed into the first) and its
+    slot is returned (``scheduler.py:1324-1363,1656-1700``); the devices' partials meet at the owner
+    of their block through the output exchange ``O``.
+    Input slots are recycled as in the reference's scheduler (``scheduler.py:826-857,2167-2199``
+    with the first-free rule of ``block_table.py:434-460``): an input block is live on a device
+    from the first to the last stage that uses it there (a work unit reads it, it arrives for
+    that stage, or it is sent for the next one), its slot is returned after the last such stage
+    has been computed, and blocks that arrive later take the lowest free slot.
+    Returns ``(fw_plans, bw_plans, layouts)`` as the unstaged builder."""
     from types import SimpleNamespace
 
     from dcp_amd.core.pipeline import generate_pipelines_n_stages
@@ -480,6 +488,20 @@ def build_staged_multi_device_plans(
             n_stages, set(devices), unit_cost, unit_inputs, meta, input_sizes, unit_device, input_device, is_bw,
             disable_two_phase_comm=disable_two_phase_comm)
 
+        # ---- how long a device needs each input block (scheduler.py:826-857) --------------------
+        last_live: List[Dict[int, int]] = [defaultdict(int) for _ in range(n_dev)]  # input id -> last stage it is live in
+        for stage_id, stage in enumerate(work_per_stage):
+            for d, ws in stage.items():
+                for w in ws:
+                    for i in unit_inputs[w]:
+                        last_live[rank_of(d)][i] = max(last_live[rank_of(d)][i], stage_id)
+        for phase in (first_phase, second_phase):
+            for stage_id, per_dst in enumerate(phase):
+                for dst, comms in per_dst.items():
+                    for i, src in comms:
+                        last_live[rank_of(dst)][i] = max(last_live[rank_of(dst)][i], stage_id)
+                        last_live[rank_of(src)][i] = max(last_live[rank_of(src)][i], stage_id - 1)
+
         # ---- per device: where each block it holds sits ----------------------------------------
         slots = [{t: _Slots() for t in ("Q", "KV", "O", "out", "dq", "dkv")} for _ in range(n_dev)]
         held: List[Dict[int, BufferBlock]] = [{} for _ in range(n_dev)]  # input id -> the block to read it from
@@ -500,6 +522,18 @@ def build_staged_multi_device_plans(
         def local_block(r, i):
             kind, g, s, b = inputs[i]
             return block_of(i, _LOCAL[kind], local_index[r][("kv" if kind == "KV" else "q", g, s, b)])
+
+        def release_dead_inputs(r, stage_id):
+            """After stage ``stage_id`` has been computed: the slots of the inputs the device needs no longer
+            (scheduler.py:2167-2199).  OUT / LSE / dOUT of a q block live and die together and share one index."""
+            for i in [i for i in held[r] if last_live[r][i] <= stage_id]:
+                kind, g, s, b = inputs[i]
+                block = held[r].pop(i)
+                if kind in ("OUT", "LSE", "dOUT"):
+                    if not any(inputs[j][0] in ("OUT", "LSE", "dOUT") and inputs[j][1:] == (g, s, b) for j in held[r]):
+                        slots[r]["O"].free(o_slot[r].pop((g, s, b)))
+                else:
+                    slots[r][kind].free(block.index)
 
         instrs: List[list] = [[] for _ in range(n_dev)]
         used = [set() for _ in range(n_dev)]  # inputs some work unit on the device reads
@@ -555,16 +589,27 @@ def build_staged_multi_device_plans(
                 return BufferBlock(buffer_type, slot, n_tok(k[1], k[2]))
 
             if not is_bw:
-                out_tab, lse_tab = [], []
+                out_tab, lse_tab, folds = [], [], []
                 for k, _ in rows:
                     slot = slots[r]["out"].take()
-                    partial_out[r][k].append(slot)
                     out_tab.append([row_block(BufferType.BUFFER_OUT, slot, k)])
                     lse_tab.append([row_block(BufferType.BUFFER_LSE, slot, k)])
+                    if partial_out[r][k]:
+                        # the block has a partial from an earlier stage: fold the new one into it and
+                        # give the new one's slot back (scheduler.py:1324-1363)
+                        old = partial_out[r][k][0]
+                        pair = lambda sl: (row_block(BufferType.BUFFER_OUT, sl, k), row_block(BufferType.BUFFER_LSE, sl, k))
+                        folds.append((ReductionOp([pair(old), pair(slot)], pair(old)), slot))
+                    else:
+                        partial_out[r][k].append(slot)
                 instrs[r].append(AttnInstr(stage_id, seq_q, seq_kv, block_size, max(seq_kv), m, q_tab, kv_tab, out_tab, lse_tab))
+                if folds:
+                    instrs[r].append(AttnReductionInstr([op for op, _ in folds], output_is_unpadded=0))
+                    for _, slot in folds:
+                        slots[r]["out"].free(slot)
                 return
             o_tab = [[row_block(BufferType.BUFFER_OUT, o_slot[r][k], k)] for k, _ in rows]
-            dq_tab, dkv_tab = [], []
+            dq_tab, dkv_tab, touched = [], [], []
             for k, ids in rows:
                 slot = slots[r]["dq"].take()
                 partial_dq[r][k].append(slot)
@@ -573,10 +618,27 @@ def build_staged_multi_device_plans(
                 for j in ids:
                     kk = (k[0] // q_per_kv, k[1], j)
                     slot = slots[r]["dkv"].take()
+                    if kk not in touched:
+                        touched.append(kk)
                     replicas[r][kk].append(slot)
                     row.append(row_block(BufferType.BUFFER_dKV, slot, kk))
                 dkv_tab.append(row)
             instrs[r].append(AttnBackwardInstr(stage_id, seq_q, seq_kv, block_size, max(seq_kv), m, q_tab, kv_tab, o_tab, dq_tab, dkv_tab))
+            # what the stage added to blocks that already had a partial, and all of a kv block's private
+            # replicas, are summed into the oldest slot and their slots given back (scheduler.py:1656-1700)
+            sums, freed = [], []
+            for what, table, keys, buffer_type in (("dq", partial_dq[r], [k for k, _ in rows], BufferType.BUFFER_dQ),
+                                                   ("dkv", replicas[r], touched, BufferType.BUFFER_dKV)):
+                for key in keys:
+                    sl = table[key]
+                    if len(sl) > 1:
+                        sums.append(SumOp([row_block(buffer_type, s_, key) for s_ in sl], row_block(buffer_type, sl[0], key)))
+                        freed += [(what, s_) for s_ in sl[1:]]
+                        del sl[1:]
+            if sums:
+                instrs[r].append(SumInstr(sums, output_is_unpadded=0))
+                for what, s_ in freed:
+                    slots[r][what].free(s_)
 
         # ---- stages: the transfers of stage k+1 are launched before stage k is computed ---------
         for k in range(n_stages + 1):
@@ -610,6 +672,7 @@ def build_staged_multi_device_plans(
             # (held already names the stage k+1 arrivals, but no work unit of stage k uses them)
             for r in range(n_dev):
                 compute(r, k)
+                release_dead_inputs(r, k)
                 for key in waits[r]:
                     instrs[r].append(CommWaitInstr(key))
 

@@ -19,6 +19,8 @@ merged (summed) exactly as partials received from other devices would be.
 
 from __future__ import annotations
 
+import heapq
+
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -147,14 +149,23 @@ class LocalLayout:
 
 
 class _Slots:
-    """First-free slot allocator of one padded buffer."""
+    """First-free slot allocator of one padded buffer: ``take`` hands out the lowest slot that is
+    not in use, ``free`` returns one (the allocation rule of the reference's BlockManager,
+    dcp/core/block_table.py:434-460).  ``n`` = slots the buffer needs."""
 
     def __init__(self):
         self.n = 0
+        self._free: List[int] = []
 
     def take(self) -> int:
+        if self._free:
+            return heapq.heappop(self._free)
         self.n += 1
         return self.n - 1
+
+    def free(self, index: int) -> None:
+        assert 0 <= index < self.n and index not in self._free, f"slot {index} is not in use"
+        heapq.heappush(self._free, index)
 
 
 def _row_ranges(seq_mask: np.ndarray, q0: int, n_q: int, block_size: int,

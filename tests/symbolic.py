@@ -34,13 +34,31 @@ class SymbolicDevice:
         for i, (g, s, b, n) in enumerate(layout.kv_blocks):
             self.slots["LocalKV"][i] = ("KV", g, s, b)
         self.pending = {}
+        # slot recycling: what every slot has held, in order, and how often each content was read,
+        # so that a read of recycled contents can say what happened and the run can report reuse
+        self.history = defaultdict(list)  # (buffer type, index) -> [name, ...]
+        self.overwritten = 0              # writes that replaced contents of another block
 
     def get(self, block):
         assert block.index < len(self.slots[block.buffer_type]), f"{block} outside its buffer"
         return self.slots[block.buffer_type][block.index]
 
+    def expect(self, block, name):
+        """A read that must find ``name``: fails with the slot's history when the slot was recycled
+        (overwritten while the block was still live) or never filled."""
+        got = self.get(block)
+        if got != name:
+            past = self.history[(block.buffer_type, block.index)]
+            why = "was overwritten while still live" if name in past else "was never put there"
+            raise AssertionError(f"{block} should hold {name} but holds {got}: it {why} (slot history {past})")
+        return got
+
     def put(self, block, name):
         assert block.index < len(self.slots[block.buffer_type]), f"{block} outside its buffer"
+        old = self.slots[block.buffer_type][block.index]
+        if old is not None and old[:4] != name[:4]:
+            self.overwritten += 1
+        self.history[(block.buffer_type, block.index)].append(name)
         self.slots[block.buffer_type][block.index] = name
 
 
@@ -84,6 +102,7 @@ def _attention(dev, instr, group_of, backward):
         assert q[0] == "Q"
         _, g, s, i = q
         kv_ids = []
+        dev.expect(q_block, q)
         assert instr.seqlens_kv[b] == bs * len(instr.kv_block_table[b])
         for kv_block in instr.kv_block_table[b]:
             assert kv_block.buffer_type == "BufferKV"
@@ -100,9 +119,9 @@ def _attention(dev, instr, group_of, backward):
             dev.put(o_block, ("out", g, s, i, frozenset(kv_ids)))
             dev.put(l_block, ("lse", g, s, i, frozenset(kv_ids)))
             continue
-        assert dev.get(o_block) == ("OUT", g, s, i), f"backward row of {q} reads {dev.get(o_block)} as its output"
-        assert dev.slots["BufferLSE"][o_block.index] == ("LSE", g, s, i)
-        assert dev.slots["BufferdOut"][o_block.index] == ("dOUT", g, s, i)
+        dev.expect(o_block, ("OUT", g, s, i))
+        dev.expect(type(o_block)("BufferLSE", o_block.index, o_block.n_tokens), ("LSE", g, s, i))
+        dev.expect(type(o_block)("BufferdOut", o_block.index, o_block.n_tokens), ("dOUT", g, s, i))
         (dq_block,) = instr.dq_block_table[b]
         assert dq_block.buffer_type == "BufferdQ" and dq_block.n_tokens == q_block.n_tokens
         dev.put(dq_block, ("dq", g, s, i, frozenset(kv_ids)))

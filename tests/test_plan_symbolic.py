@@ -49,6 +49,54 @@ def test_multi_device_plans(name):
         run_symbolic(plans, case["layouts"], case["n_devices_per_node"], backward, case["mask"], _q_per_kv(cfg))
 
 
+def test_staged_plans_recycle_slots_and_no_live_block_is_overwritten():
+    """The staged builder returns the slots of input blocks after the last stage that needs them and
+    of partials once they are folded (the reference's BlockManager with live ranges): the symbolic run,
+    which follows every slot's contents through time, passes, it sees slots change hands, and the
+    buffers are smaller than one slot per block ever held."""
+    cfg = MULTI["staged_four_stages"]
+    case = make_multi_case(**cfg)
+    for plans, backward in ((case["fw"], False), (case["bw"], True)):
+        devs = run_symbolic(plans, case["layouts"], case["n_devices_per_node"], backward, case["mask"], _q_per_kv(cfg))
+        assert sum(d.overwritten for d in devs) > 0, "no slot was recycled"
+        saved = 0
+        for plan in plans:
+            n_kv_writes = sum(1 for i in plan.instructions if isinstance(i, CommLaunchInstr)
+                              for op in i.comm_ops if op.comm_type == 1 and op.buffer_block.buffer_type == "BufferKV")
+            n_kv_writes += sum(1 for i in plan.instructions if type(i).__name__ == "MemcpyInstr"
+                               for _, dst in i.src_dst_pairs if dst.buffer_type == "BufferKV")
+            saved += n_kv_writes - plan.buffer_info["BufferKV"].n_blocks
+        assert saved > 0, "every kv block ever held still has a slot of its own"
+
+
+def test_the_checker_notices_a_slot_recycled_too_early():
+    """A receive redirected into a slot whose block a later stage still reads is reported as such."""
+    cfg = MULTI["staged_four_stages"]
+    case = make_multi_case(**cfg)
+    plans = case["fw"]
+    # the first kv block some device receives goes, instead of to its slot, to the slot of a block
+    # that the device gathered at the start and reads in a later stage
+    for plan in plans:
+        attn_stages = [i for i in plan.instructions if type(i).__name__ == "AttnInstr"]
+        launch = next((i for i in plan.instructions if isinstance(i, CommLaunchInstr)
+                       and any(op.comm_type == 1 and op.buffer_block.buffer_type == "BufferKV" for op in i.comm_ops)), None)
+        if launch is None or len(attn_stages) < 2:
+            continue
+        k = next(n for n, op in enumerate(launch.comm_ops) if op.comm_type == 1 and op.buffer_block.buffer_type == "BufferKV")
+        victim = attn_stages[0].kv_block_table[0][0]  # read by the stage that runs while this transfer is in flight
+        op = launch.comm_ops[k]
+        if victim.n_tokens != op.buffer_block.n_tokens or victim.index == op.buffer_block.index:
+            continue
+        launch.comm_ops[k] = CommOp(op.comm_type, op.peer, BufferBlock("BufferKV", victim.index, victim.n_tokens))
+        # the stage after the wait reads the victim's slot again only if it is still live there; make it so
+        attn_stages[1].kv_block_table[0][0] = victim
+        break
+    else:
+        pytest.skip("no device of this case both receives kv blocks and runs two stages")
+    with pytest.raises(AssertionError):
+        run_symbolic(plans, case["layouts"], case["n_devices_per_node"], False, case["mask"], _q_per_kv(cfg))
+
+
 def test_the_checker_notices_a_wrong_plan():
     """A kv block swapped in an attention row, a receive into the wrong kind of slot and a dropped
     work unit must each fail."""
