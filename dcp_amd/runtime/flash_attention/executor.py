@@ -299,17 +299,19 @@ class DCPAttention(torch.autograd.Function):
 
 
 def _prepare_memcpy(exec: AttentionExecutor, instr: MemcpyInstr):
-    """One argument table per (dtype, block numel) for data blocks and one for
-    LSE blocks.  The source is the unpadded buffer, addressed by
-    ``local_cu_seqlens`` (reference ``_prepare_memcpy`` :606-790)."""
+    """One argument table per dtype for data blocks and one for LSE blocks.  The source is the
+    unpadded buffer, addressed by ``local_cu_seqlens`` (reference ``_prepare_memcpy`` :606-790,
+    which makes one table, and one launch, per (dtype, block numel): here blocks of different
+    sizes share a launch, whose grid is sized for the largest -- every block carries its own
+    element count and stride, and the workgroups past a smaller block's end leave at once)."""
     cu = exec.execution_plan.local_cu_seqlens
     data = defaultdict(lambda: [[] for _ in range(7)])
     lse = defaultdict(lambda: [[] for _ in range(7)])
     head_block_size = None
     for src, dst in instr.src_dst_pairs:
         src_buf, dst_buf = exec.buffers[src.buffer_type], exec.buffers[dst.buffer_type]
-        key = (src_buf.dtype, exec.buffer_block_strides[src.buffer_type])
         src_off = cu[src.index]
+        key = (src_buf.dtype, exec.buffer_block_strides[src.buffer_type]) if src.buffer_type in _LSE_BUFFER_TYPES else src_buf.dtype
         if src.buffer_type in _LSE_BUFFER_TYPES:
             assert dst.buffer_type in _LSE_BUFFER_TYPES
             cols = lse[key]
@@ -343,7 +345,8 @@ def _prepare_memcpy(exec: AttentionExecutor, instr: MemcpyInstr):
         return tuple(_dev(c, k) for c, k in zip(cols, kinds))
 
     exec._args_cache[exec.instr_index] = {
-        "other": {key: tables(cols) for key, cols in data.items()},
+        # key: (dtype, the largest block numel of the launch)
+        "other": {(dtype, max(cols[5])): tables(cols) for dtype, cols in data.items()},
         "lse": {key: tables(cols) + (head_block_size,) for key, cols in lse.items()},
     }
 
@@ -582,11 +585,12 @@ def _handle_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
 def _prepare_sum(exec: AttentionExecutor, instr: SumInstr):
     groups = defaultdict(lambda: defaultdict(list))
     cu = exec.execution_plan.local_cu_seqlens
+    # one launch per dtype: sums over blocks of different sizes share it (its grid is sized for the
+    # largest block, every sum carries its own element count and strides)
     for op in instr.ops:
         src_type = op.src_buffers[0].buffer_type
         dst_type = op.dst_buffer.buffer_type
-        key = (exec.buffers[src_type].dtype, exec.buffer_block_strides[src_type])
-        g = groups[key]
+        g = groups[exec.buffers[src_type].dtype]
         per_token = int(np.prod(exec.buffer_per_token_shape[src_type]))
         g["src_ptrs"].append(exec.buffers[src_type].data_ptr())
         g["src_offsets"].append([blk.index for blk in op.src_buffers])
@@ -601,10 +605,10 @@ def _prepare_sum(exec: AttentionExecutor, instr: SumInstr):
             g["dst_strides"].append(exec.buffer_block_strides[dst_type])
         g["n_elems"].append(op.dst_buffer.n_tokens * per_token)
     prepared = {}
-    for key, g in groups.items():
+    for dtype, g in groups.items():
         width = _round_to_pow_2(max(g["n_ops"]))
         padded = [row + [-1] * (width - len(row)) for row in g["src_offsets"]]
-        prepared[key] = (
+        prepared[(dtype, max(g["src_strides"]))] = (
             _dev(g["src_ptrs"], torch.int64),
             _dev(padded, torch.int32),
             _dev(g["src_strides"], torch.int32),
