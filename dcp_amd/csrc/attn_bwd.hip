@@ -269,6 +269,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   const uint32_t goff0 = Tile::lane_offset0(q_row_stride, w, lane);
   // tile load idx of a step: the wave's group loads of the Q tile, then of the dO tile
   constexpr int NL = 2 * Tile::LPW;
+  const uint64_t group_step = uniform64(Tile::group_global_step(q_row_stride));
   static_assert(NL <= KS, "a sub-step carries half of the tile loads, one per two k-steps of its first phase");
   auto request_tile = [&](int idx, int head, int qt, int st) {
     const int64_t off = (int64_t)qt * BM * q_row_stride + (int64_t)head * D;
@@ -329,6 +330,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     const int qt_next = more ? __builtin_ctzll(rem) : qt;
     const uint16_t* q_lds = tiles[2 * st];
     const uint16_t* do_lds = tiles[2 * st + 1];
+    // where the next step's tiles come from and go to, as wave-uniform scalars worked out once a
+    // step: a load in the matrix phases then costs two scalar additions
+    const int64_t off_next = (int64_t)qt_next * BM * q_row_stride + (int64_t)head_next * D;
+    const uint64_t next_q = uniform64(reinterpret_cast<uint64_t>(q_base + off_next));
+    const uint64_t next_do = uniform64(reinterpret_cast<uint64_t>(do_base + off_next));
+    const uint32_t next_at = __builtin_amdgcn_readfirstlane(Tile::group_lds_at(tiles_at + 2 * (st ^ 1) * (Tile::SIZE * 2), w, 0));
 
     // One sub-step = this wave's 32 keys against 32 of the step's 64 queries (QI = 0, 1).
     // (A real loop, not unrolled: one copy of the body keeps the register allocation of a single
@@ -389,6 +396,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         const int i = o - N1, s2 = i / (2 * DT), d = (i % (2 * DT)) / 2;
         return Tile::template read_col<true>((i & 1) ? q_lds : do_lds, col_rd_q, s2, d);
       };
+      // this sub-step's half of the next step's tile loads: the Q tile (QI = 0) or the dO tile
+      static_assert(NL / 2 == Tile::LPW, "a sub-step loads one whole tile");
+      uint64_t load_src = uniform64(QI ? next_do : next_q);
+      const uint32_t load_at = next_at + QI * (Tile::SIZE * 2);
       u32x4 buf[RING];
 #pragma unroll
       for (int o = 0; o < AHEAD; ++o) buf[o] = entry(o);
@@ -406,7 +417,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         // first operand of the second phase is requested before the vector phase (registers)
         if (o + AHEAD < N1 + PRE) buf[(o + AHEAD) % RING] = entry(o + AHEAD);
         // this sub-step's half of the next step's tile loads, one per two k-steps
-        if (kind == 2 && ks % 2 == 0 && ks / 2 < NL / 2) request_tile(QI * (NL / 2) + ks / 2, head_next, qt_next, st ^ 1);
+        if (kind == 2 && ks % 2 == 0 && ks / 2 < NL / 2) {
+          Tile::load_group_at(load_at + (ks / 2) * (Tile::GROUP_STRIDE * 2), load_src, goff0);
+          load_src = uniform64(load_src + group_step);
+        }
         __builtin_amdgcn_sched_barrier(0);  // keeps the order: reads neither pile up in registers nor fall behind
       }
       // ---- P = exp2(S c - lse), dS = P (dP - delta), packed in accumulator order: as B operands

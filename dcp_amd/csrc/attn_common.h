@@ -154,6 +154,12 @@ __device__ __forceinline__ void load_async_dword(uint32_t lds_at, uint32_t lane_
                : "memory");
 }
 
+// A 64-bit value that every lane holds alike, moved to scalar registers.
+__device__ __forceinline__ uint64_t uniform64(uint64_t a) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
 template <int D, int NW = 4>
 struct KvTile {
   static constexpr int ROWS = 64;
@@ -231,6 +237,20 @@ struct KvTile {
                  : "s"(lds_at), "v"(off0), "s"(base)
                  : "memory");
   }
+  // One group load whose LDS byte address and wave-uniform global base the caller has already
+  // worked out (kernels that walk a tile's groups keep both as running scalars).
+  __device__ static __forceinline__ void load_group_at(uint32_t lds_at, uint64_t base, uint32_t off0) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_at), "v"(off0), "s"(base)
+                 : "memory");
+  }
+  // LDS byte address of the wave's group load i, and the global byte step between group loads (its
+  // rows lie four rows below those of load i - 1)
+  __device__ static __forceinline__ uint32_t group_lds_at(uint32_t tile_at, int wave, int i) {
+    return tile_at + (wave * LPW + i) * GROUP_STRIDE * 2;
+  }
+  __device__ static __forceinline__ uint64_t group_global_step(int64_t row_stride) { return (uint64_t)row_stride * 8; }
   // Row operand of lane (c, h): elements 16*ks + 8h.. of row 32*nt + c at
   //   tile + row_base(c, h) + nt*ROW32 + ks*16
   __device__ static __forceinline__ int row_base(int c, int h) { return at(c, 8 * h); }
