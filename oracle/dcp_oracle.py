@@ -6,7 +6,7 @@ A numpy restatement of what the reference computes on this path.  Each
 function cites the reference code it follows (paths relative to the reference
 repository root):
 
-  block_copy / lse_copy   commented torch fallback of _handle_memcpy
+  block_copy              commented torch fallback of _handle_memcpy
                           (dcp/runtime/flash_attention/executor.py:814-831),
                           kernels dcp/ops/fused_ops.py:290-335, 370-429
   merge_out_lse           _flash_attn_update_out_lse (fused_ops.py:15-146);
@@ -28,7 +28,8 @@ repository root):
                           CommWaitInstr) executor.py:1583-2074
 
 Pinning (tests/test_oracle.py): block movement against numpy fancy indexing
-and gather/scatter round trips; merge against scipy.special.logsumexp, the
+and gather/scatter round trips; the block sum against math.fsum (the exactly
+rounded sum) and exact integer sums; merge against scipy.special.logsumexp, the
 folded pairwise sigmoid form and its invariants; attention forward against
 torch.nn.functional.scaled_dot_product_attention and a dense boolean mask;
 backward against torch.autograd and central finite differences; masks against
@@ -84,12 +85,6 @@ def block_copy(src_flat, src_elem_offsets, dst_flat, dst_elem_offsets, n_element
     """dst[dst_off : dst_off+n] = src[src_off : src_off+n] for every pair."""
     for so, do, n in zip(src_elem_offsets, dst_elem_offsets, n_elements):
         dst_flat[do : do + n] = src_flat[so : so + n]
-
-
-def lse_copy(src, src_token_offsets, dst, dst_token_offsets, n_tokens):
-    """src, dst are [heads, tokens]-shaped 2-D views."""
-    for so, do, n in zip(src_token_offsets, dst_token_offsets, n_tokens):
-        dst[:, do : do + n] = src[:, so : so + n]
 
 
 # ---------------------------------------------------------------------------

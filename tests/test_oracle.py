@@ -53,6 +53,29 @@ def _rand_partials(seed, S=5, T=17, H=3, D=8, lo=-5.0, hi=5.0):
     return rng.standard_normal((S, T, H, D)), rng.uniform(lo, hi, (S, H, T))
 
 
+def test_blockwise_sum_is_the_exact_sum():
+    """Pinned by the exactly rounded sum (math.fsum) element by element, by integer-valued blocks
+    whose sum is exact in every order, and by order invariance on them; the single rounding to the
+    storage type is torch's (test_round_bf16_matches_torch)."""
+    import math
+
+    rng = np.random.default_rng(5)
+    srcs = [rng.standard_normal((7, 33)).astype(np.float32) * 10.0 ** rng.integers(-3, 4) for _ in range(9)]
+    got = oracle.blockwise_sum(srcs)
+    assert got.dtype == np.float64 and got.shape == (7, 33)
+    exact = np.array([[math.fsum(float(s[i, j]) for s in srcs) for j in range(33)] for i in range(7)])
+    # nine float64 additions of float32 values: within a few ulps of the exact sum's magnitude
+    assert np.abs(got - exact).max() <= 16 * np.finfo(np.float64).eps * np.abs(np.stack(srcs)).sum(0).max()
+    ints = [rng.integers(-1000, 1000, size=(5, 16)).astype(np.float32) for _ in range(6)]
+    want = np.stack(ints).astype(np.int64).sum(0)
+    assert np.array_equal(oracle.blockwise_sum(ints), want)
+    assert np.array_equal(oracle.blockwise_sum(ints[::-1]), want)
+    assert np.array_equal(oracle.blockwise_sum([ints[0]]), ints[0])  # one source: the block itself
+    # bf16 sources are summed as the values they hold, not re-rounded in between
+    b = [oracle.round_to(x * 0.37, "bf16") for x in ints]
+    assert np.array_equal(oracle.blockwise_sum(b), np.stack([np.asarray(x, np.float64) for x in b]).sum(0))
+
+
 def test_merge_against_scipy_logsumexp():
     outs, lses = _rand_partials(0)
     out, lse = oracle.merge_out_lse(outs, lses)
