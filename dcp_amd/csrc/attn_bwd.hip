@@ -195,6 +195,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // stores nothing.  Its K/V addresses fall back to the tile's first keys so that they stay valid.
   const int kw = k0 + w * 32;
   const bool has_keys = kw < seqlen_kv;
+  const int kv_or_beyond = kw + c < seqlen_kv ? kw + c : 0x7fffffff;  // this lane's key, for the range tests
   const int kw_safe = has_keys ? kw : k0;
   const int blk = __builtin_amdgcn_readfirstlane(kw_safe / p.block_size);
   const int tok0 = kw_safe - blk * p.block_size;
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
       // (A = rows of the Q / dO tile, B = K / V in registers; lane = key, element i = query
       // 32 QI + acc_row(i, h)).  The range mask enters S as the accumulator's initial value.
       f32x16 s_acc, dp_acc;
-      const int kv = kw + c;
+      const int q_left = seqlen_q - (qt * BM + QI * 32 + 4 * h);  // valid queries from this lane's first one on
       if (unmasked) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
@@ -362,10 +363,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
           for (int pl = 0; pl < 4; ++pl) rs[pl] = *reinterpret_cast<const i32x4*>(&rng_lds[st][pl][QI * 32 + 8 * g + 4 * h]);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int s0 = rs[0][r], len0 = min(rs[1][r], seqlen_kv) - s0;
-            const int s1 = rs[2][r], len1 = min(rs[3][r], seqlen_kv) - s1;
-            bool ok = ((unsigned)(kv - s0) < (unsigned)max(len0, 0)) | ((unsigned)(kv - s1) < (unsigned)max(len1, 0));
-            ok &= qt * BM + QI * 32 + 8 * g + 4 * h + r < seqlen_q;
+            // five comparisons per element and nothing else on the vector unit: a key past the
+            // row's last one counts as beyond every range (kv_or_beyond), a query past the
+            // row's last one fails its own test
+            bool ok = ((kv_or_beyond >= rs[0][r]) & (kv_or_beyond < rs[1][r])) |
+                      ((kv_or_beyond >= rs[2][r]) & (kv_or_beyond < rs[3][r]));
+            ok &= 8 * g + r < q_left;
             s_acc[4 * g + r] = ok ? 0.0f : -INFINITY;
           }
           __builtin_amdgcn_sched_barrier(0);  // one group's planes in registers at a time
@@ -677,9 +680,9 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
 #pragma unroll
         for (int i = 0; i < 16; ++i) s_acc[i] = 0.0f;
       } else {
-        const int kb = k0 + nt * 32 + 4 * h;
+        const uint32_t closed = rng.closed_window(k0 + nt * 32) >> (4 * h);  // bit = key - first key of the half
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_acc[i] = rng.contains(kb + 8 * (i / 4) + (i % 4)) ? 0.0f : -INFINITY;
+        for (int i = 0; i < 16; ++i) s_acc[i] = masked_start(closed, 8 * (i / 4) + (i % 4));
       }
       // operands four k-steps at a time; the two accumulation chains interleave
 #pragma unroll

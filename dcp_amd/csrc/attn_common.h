@@ -418,6 +418,21 @@ struct RangePair {
   __device__ __forceinline__ bool contains(int k) const {
     return ((unsigned)(k - s0) < (unsigned)len0) | ((unsigned)(k - s1) < (unsigned)len1);
   }
+  // Bit p set = key base + p (p = 0..31) lies in neither range.  A dozen vector instructions
+  // for a 32-key window, after which an accumulator's initial value costs two (masked_start)
+  // where a range test per element costs seven.
+  __device__ __forceinline__ uint32_t closed_window(int base) const {
+    auto open = [&](int s, int len) -> uint32_t {
+      const int lo = min(max(s - base, 0), 32), hi = min(max(s + len - base, lo), 32);
+      return (uint32_t)((1ull << hi) - (1ull << lo));  // bits lo..hi-1; the low word also when hi or lo is 32
+    };
+    return ~(open(s0, len0) | open(s1, len1));
+  }
 };
+// 0.0f where bit `bit` of `closed` is clear, -inf where it is set: the bit, sign-extended to 0 / -1,
+// shifted into the sign and exponent of a float.
+__device__ __forceinline__ float masked_start(uint32_t closed, int bit) {
+  return __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_sbfe((int32_t)closed, bit, 1) & 0xff800000u);
+}
 
 }  // namespace dcp

@@ -293,14 +293,16 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 #pragma unroll
           for (int e = 0; e < 16; ++e) s_out[nt][qb][e] = 0.0f;
     } else {
-      const int kb = tile * BN + 4 * h;
+      // the keys a row may not see, as a bit mask per 32-key half (bit = key - first key of the
+      // half), shifted so that element e of this lane's half h is bit 8 (e / 4) + e % 4
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
+        for (int qb = 0; qb < QB; ++qb) {
+          const uint32_t closed = rng[qb].closed_window(tile * BN + nt * 32) >> (4 * h);
 #pragma unroll
-          for (int e = 0; e < 16; ++e)
-            s_out[nt][qb][e] = rng[qb].contains(kb + nt * 32 + 8 * (e / 4) + (e % 4)) ? 0.0f : -INFINITY;
+          for (int e = 0; e < 16; ++e) s_out[nt][qb][e] = masked_start(closed, 8 * (e / 4) + (e % 4));
+        }
     }
     constexpr int N = 2 * KS, AHEAD = 3;
     u32x4 ka[4];
