@@ -42,6 +42,7 @@ from dcp_amd.core.instructions import (
     SumOp,
 )
 from dcp_amd.core.serialization import torch_dtype_to_int
+from dcp_amd.runtime.flash_attention.workload import concat_local_attn_masks, generate_work_units, rows_of_work_units
 
 
 @dataclass
@@ -232,6 +233,7 @@ def build_single_device_plans(
     kv_split: str = "round_robin",
     fold_stages: bool = False,
     backward: bool = True,
+    work_units: str = "overlap",
 ):
     """Returns ``(fw_plan, bw_plan, layout)`` (``bw_plan`` is ``None`` when
     ``backward`` is false).
@@ -242,7 +244,14 @@ def build_single_device_plans(
     ``n_kv_groups``/``kv_split`` split each row's kv blocks into partials;
     ``fold_stages`` merges each later stage's partial into the stage-0 partial
     in place (padded destination) instead of one N-way merge at the end.
+    ``work_units`` chooses which (q block, kv block) pairs a row holds:
+    ``"overlap"`` keeps the pairs in which some query attends some key;
+    ``"reference"`` goes the reference's way through block-local masks
+    (``workload.generate_work_units`` / ``concat_local_attn_masks``), which also
+    keeps pairs that only the hull of the block's ranges touches (all their
+    ranges are empty; same results, a few more kv blocks per row).
     """
+    assert work_units in ("overlap", "reference")
     raw_seqlens = [int(x) for x in raw_seqlens]
     assert n_heads % n_query_groups == 0
     group = n_heads // n_query_groups
@@ -308,11 +317,19 @@ def build_single_device_plans(
         kv_ids: List[int]
 
     rows: List[Row] = []
+    local_masks: Dict[Tuple[int, int, int], np.ndarray] = {}  # (sequence, q block, kv block), "reference" only
     for s, L in enumerate(raw_seqlens):
         seq_mask = mask_np[seq_off[s] : seq_off[s + 1]]
+        if work_units == "reference":
+            units = generate_work_units(seq_mask, L, block_size)
+            local_masks.update({(s, i, j): m for (i, j), m in units.items()})
+            kv_of = rows_of_work_units(units)
         for b in range(n_blocks_of[s]):
-            kv_ids = _block_overlaps(seq_mask, b * block_size, n_tok(s, b), block_size,
-                                     n_blocks_of[s], L)
+            if work_units == "reference":
+                kv_ids = kv_of.get(b, [])
+            else:
+                kv_ids = _block_overlaps(seq_mask, b * block_size, n_tok(s, b), block_size,
+                                         n_blocks_of[s], L)
             for g in range(n_hb_q):
                 rows.append(Row(g, s, b, kv_ids))
     rows.sort(key=lambda r: (r.s, r.g, r.b))
@@ -341,6 +358,13 @@ def build_single_device_plans(
         planes = []
         for r, ids in stage_rows:
             seq_mask = mask_np[seq_off[r.s] : seq_off[r.s + 1]]
+            if work_units == "reference":
+                joined = concat_local_attn_masks([local_masks[(r.s, r.b, j)] for j in ids],
+                                                 [n_tok(r.s, j) for j in ids], n_tok(r.s, r.b))
+                plane = np.zeros(joined.shape[:2] + (block_size,), dtype=np.int32)
+                plane[..., : joined.shape[2]] = joined
+                planes.append(plane)
+                continue
             planes.append(
                 _row_ranges(seq_mask, r.b * block_size, n_tok(r.s, r.b), block_size, ids,
                             [n_tok(r.s, j) for j in ids])

@@ -44,11 +44,12 @@ def check_against_truth(res, truth, out_tol=OUT_TOL):
 
 def make_case(seqlens, block_size, n_heads, n_groups, head_dim, head_block, mask="causal",
               mask_info=None, dtype="bf16", n_kv_groups=1, kv_split="round_robin", fold=False,
-              seed=0, qkv_scale=1.0, mask_kwargs=None):
+              seed=0, qkv_scale=1.0, mask_kwargs=None, work_units="overlap"):
     mask_t = MASK_FNS[mask](list(seqlens), list(seqlens), torch.int32, mask_info, **(mask_kwargs or {}))
     fw, bw, layout = build_single_device_plans(
         seqlens, block_size, n_heads, n_groups, head_dim, head_block, mask_t,
-        dtype=TORCH_DTYPE[dtype], n_kv_groups=n_kv_groups, kv_split=kv_split, fold_stages=fold)
+        dtype=TORCH_DTYPE[dtype], n_kv_groups=n_kv_groups, kv_split=kv_split, fold_stages=fold,
+        work_units=work_units)
     g = torch.Generator().manual_seed(seed)
     T = sum(seqlens)
     q = (torch.randn(T, n_heads, head_dim, generator=g) * qkv_scale).to(TORCH_DTYPE[dtype])
