@@ -98,6 +98,22 @@ def _check_tables(batch, cu_seqlens_k, row_order, single, wide):
         raise ValueError(f"row_order must have {batch} entries, got {row_order.numel()}")
 
 
+KERNEL_HEAD_DIMS = (64, 128)
+
+
+def _kernel_head_dim(head_dim: int) -> int:
+    """The head size the kernels run a given head size at."""
+    for d in KERNEL_HEAD_DIMS:
+        if head_dim <= d:
+            return d
+    raise ValueError(f"head size {head_dim} is above the largest supported one ({KERNEL_HEAD_DIMS[-1]})")
+
+
+def _widen(t: torch.Tensor, d: int) -> torch.Tensor:
+    """A dense copy of ``t`` with its last axis zero-padded to ``d``."""
+    return torch.nn.functional.pad(t, (0, d - t.shape[-1]))
+
+
 def _range_arg(attn_range: torch.Tensor, total_q: int):
     _i32(attn_range, "attn_range")
     if attn_range.dim() == 2 and tuple(attn_range.shape) == (2, total_q):
@@ -168,6 +184,19 @@ def _flash_attn_varlen_forward(
         raise ValueError(f"lse_ shape {tuple(lse_.shape)} does not match out_")
     if softmax_scale is None:
         softmax_scale = head_dim ** (-0.5)
+    if head_dim not in KERNEL_HEAD_DIMS:
+        # Any other head size runs at the next kernel head size on zero-padded copies, like the
+        # reference pads head sizes that are not multiples of 8 (dcp/runtime/flash_attention/
+        # executor.py:156-160): zero columns add nothing to a score, and the scale is already
+        # fixed.  A compatibility path: it allocates and copies whole buffers on every call.
+        d = _kernel_head_dim(head_dim)
+        out_wide = _widen(out_, d)  # carries the slots this call does not write
+        _flash_attn_varlen_forward(
+            _widen(q, d), _widen(k, d), _widen(v, d), cu_seqlens_q, cu_seqlens_k, total_q, max_seqlen_q, max_seqlen_k,
+            dropout_p, softmax_scale, attn_range=attn_range, q_block_table=q_block_table, kv_block_table=kv_block_table,
+            out_block_table=out_block_table, out_=out_wide, lse_=lse_, row_order=row_order, workspace=workspace)
+        out_.copy_(out_wide[..., :head_dim])
+        return out_, lse_, None, None
     if workspace is None:
         workspace = forward_workspace(q.device)
     if workspace.dtype != torch.int32 or not workspace.is_contiguous():
@@ -264,6 +293,21 @@ def _flash_attn_varlen_backward(
         raise ValueError("dout and out must have the same number of slots")
     if softmax_scale is None:
         softmax_scale = head_dim ** (-0.5)
+    if head_dim not in KERNEL_HEAD_DIMS:
+        # as in the forward: zero-padded copies at the next kernel head size; the gradients'
+        # padded columns come out zero and are dropped, slots this call leaves alone are carried
+        d = _kernel_head_dim(head_dim)
+        dq_wide, dk_wide, dv_wide = _widen(dq, d), _widen(dk, d), _widen(dv, d)
+        _flash_attn_varlen_backward(
+            _widen(dout, d), _widen(q, d), _widen(k, d), _widen(v, d), _widen(out, d), softmax_lse, dq_wide, dk_wide,
+            dv_wide, cu_seqlens_q, cu_seqlens_k, total_q, total_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
+            causal, window_size_left, window_size_right, softcap, alibi_slopes, deterministic, attn_range=attn_range,
+            q_block_table=q_block_table, kv_block_table=kv_block_table, out_block_table=out_block_table,
+            dq_block_table=dq_block_table, dkv_block_table=dkv_block_table, workspace=workspace, row_order=row_order)
+        dq.copy_(dq_wide[..., :head_dim])
+        dk.copy_(dk_wide[..., :head_dim])
+        dv.copy_(dv_wide[..., :head_dim])
+        return dq, dk, dv, None
     need = backward_workspace_bytes(batch, int(total_q), block_size, n_heads_q, head_dim)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)

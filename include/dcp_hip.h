@@ -177,7 +177,10 @@ int dcp_blockwise_sum(const int64_t* src_ptrs, const int32_t* src_offsets,
  * the order in which they are scheduled (put the rows with most keys first);
  * NULL = as numbered.  It changes no result.
  * Supported: dtype bf16/fp16, head_dim 64 or 128, block_size % 64 == 0,
- * softmax_scale > 0.
+ * softmax_scale > 0.  (A caller with another head size up to 128 zero-pads its
+ * buffers to the next of the two and keeps its own softmax_scale, as the
+ * reference pads head sizes its kernels do not take; the Python operator layer
+ * does so.)
  * Key/value tiles are loaded whole: what a slot holds past the row's keys (and,
  * for keys a range excludes, inside it) reaches the matrix instructions and is
  * masked there.  It must be finite, and small enough that its dot products with

@@ -91,6 +91,17 @@ def test_forward_matches_plan_oracle_buffers(gpu):
     assert np.abs(res[1].numpy() - ref[1].numpy()).max() <= LSE_TOL
 
 
+# Head sizes the kernels are not built for run zero-padded at the next one that is (64, 128), as
+# the reference pads head sizes to what its kernels take: multiples of 8 and one that is not.
+FWD_CASES.update({
+    "head_dim_96": dict(seqlens=[300, 77], block_size=128, n_heads=4, n_groups=2, head_dim=96, head_block=2,
+                        n_kv_groups=2),
+    "head_dim_40": dict(seqlens=[200], block_size=64, n_heads=2, n_groups=2, head_dim=40, head_block=2,
+                        mask="lambda", mask_kwargs=dict(n_starting=8, l_pretrain=50)),
+    "head_dim_100_fp16": dict(seqlens=[150, 40], block_size=64, n_heads=2, n_groups=1, head_dim=100, head_block=2,
+                              dtype="fp16"),
+})
+
 BWD_CASES = {
     "causal_d64": dict(seqlens=[512, 300], block_size=256, n_heads=4, n_groups=4, head_dim=64, head_block=2),
     "gqa_ragged_d128": dict(seqlens=[1000, 333, 1, 257], block_size=256, n_heads=8, n_groups=2,
@@ -110,6 +121,9 @@ BWD_CASES = {
     "multimodal_image_to_self": FWD_CASES["multimodal_image_to_self"],
     "shared_question": FWD_CASES["shared_question"],
     "tiny_blocks": FWD_CASES["tiny_blocks"],
+    "head_dim_96": dict(FWD_CASES["head_dim_96"], qkv_scale=0.5),
+    "head_dim_40": dict(FWD_CASES["head_dim_40"], qkv_scale=0.5),
+    "head_dim_100_fp16": dict(FWD_CASES["head_dim_100_fp16"], qkv_scale=0.5),
 }
 
 
