@@ -287,6 +287,26 @@ def movement_microbench(iters=5, bs=512):
     n, total = _lib.profile_report()["copy_varlen_kernel"]
     copy_bytes = 2 * tokens * heads * d * 2
     copy_gbps = copy_bytes / (total / n * 1e-3) / 1e9
+
+    # the same bytes as one-head blocks (head block size 1: 16384 blocks of 128 KiB)
+    n1, numel1 = n_blocks * heads, bs * d
+    perm1 = rng.permutation(n1)
+    ident1, stride1 = np.arange(n1), i32([numel1] * n1)
+    gather1 = (i64([src.data_ptr()] * n1), i32(ident1), stride1, i64([packed.data_ptr()] * n1), i32(perm1), stride1, stride1)
+    scatter1 = (i64([packed.data_ptr()] * n1), i32(perm1), stride1, i64([back.data_ptr()] * n1), i32(ident1), stride1, stride1)
+    back.zero_()
+    fused_copy_bf16_varlen(*gather1, numel1, 128)
+    fused_copy_bf16_varlen(*scatter1, numel1, 128)
+    torch.cuda.synchronize()
+    exact = exact and bool(torch.equal(back, src))
+    _lib.profile_enable(True)
+    for _ in range(iters):
+        fused_copy_bf16_varlen(*gather1, numel1, 128)
+        fused_copy_bf16_varlen(*scatter1, numel1, 128)
+    torch.cuda.synchronize()
+    _lib.profile_enable(False)
+    n, total = _lib.profile_report()["copy_varlen_kernel"]
+    copy1_gbps = copy_bytes / (total / n * 1e-3) / 1e9
     del packed, back
 
     # merge: 4 partial outs per q block
@@ -339,9 +359,10 @@ def movement_microbench(iters=5, bs=512):
         torch.cuda.synchronize()
         stream_gbps[ns] = (ns + 1) * per_stream / (e0.elapsed_time(e1) / iters * 1e-3) / 1e9
     return dict(
-        workload="block movement: 262144 tok x 32 heads x 128 bf16, 512-token blocks, seeded permutation",
+        workload="block movement: 262144 tok x 32 heads x 128 bf16, 512-token blocks (512 blocks of 4 MiB; as one-head blocks 16384 of 128 KiB), seeded permutation",
         gather_scatter_GBps=round(copy_gbps, 1),
         gather_scatter_frac_of_8TBps=round(copy_gbps / PEAK_HBM_GBPS, 4),
+        gather_scatter_one_head_blocks_GBps=round(copy1_gbps, 1),
         gather_scatter_roundtrip_bit_exact=exact,
         copy_bytes_per_launch=copy_bytes,
         merge4_GBps=round(merge_gbps, 1),

@@ -164,6 +164,26 @@ def test_config2_llama_shape_sampled_parity_linearity_determinism(gpu):
     assert torch.equal(t[B.LOCAL_dQ], dq0 * 2) and torch.equal(t[B.LOCAL_dKV], dkv0 * 2)
 
 
+def test_config2_four_stage_round_robin_variant(gpu):
+    """The same 65536-token schedule with every row's kv blocks dealt round-robin to four stages:
+    four partial outputs per row merged at the end (N-way merge with up to four sources), dQ summed
+    over the stages' versions, dK/dV replicas per (row, kv block) as before."""
+    from dcp_amd.core.instructions import AttnReductionInstr, BufferType as B, SumInstr
+
+    wl = dict(bench.workload("llama3_8b_causal_64k"), plan_kwargs=dict(n_kv_groups=4, kv_split="round_robin"))
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl, seed=6)
+    reds = [i for i in fw.instructions if isinstance(i, AttnReductionInstr)]
+    assert max(len(op.src_buffers) for r in reds for op in r.ops) == 4
+    sums = [i for i in bw.instructions if isinstance(i, SumInstr)]
+    assert max(len(op.src_buffers) for r in sums for op in r.ops if op.dst_buffer.buffer_type == B.BUFFER_dQ) == 4
+    order = np.argsort(wl["seqlens"])
+    worst = _sample_check(wl, layout, mask, t, [(int(order[1]), 2)])
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+    s = int(np.argmax(wl["seqlens"]))  # the longest sequence: rows with the most kv blocks per stage
+    worst = _dense_check_gpu(wl, mask, t, s, kvh=4)
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+
+
 def test_config2_hip_graph_replays_match_eager(gpu):
     from dcp_amd.core.instructions import BufferType as B
     from dcp_amd.runtime.flash_attention.executor import get_executor
@@ -283,6 +303,43 @@ def test_config4_shared_prefix_full_size_dense_check(gpu):
     want = sum(i["prefix"] * (i["prefix"] + 1) // 2 + sum(c * i["prefix"] + c * (c + 1) // 2 for c in i["continuations"])
                for i in wl["mask_info"])
     assert count_attended_pairs(mask) == want
+
+
+def test_config4_head_block_of_one(gpu):
+    """Config 4 with one q head per head block (five head blocks per kv head): the dK/dV sum then
+    adds the replicas of five q head blocks."""
+    wl = dict(bench.workload("shared_prefix_96k"), head_block=1)
+    fw, bw, layout, mask, ex_f, ex_b, t = _run(wl, seed=7)
+    s = int(np.argmin(wl["seqlens"]))
+    worst = _dense_check_gpu(wl, mask, t, s, kvh=5)
+    assert worst["out"] <= 2e-2 and worst["lse"] <= 1e-3 and worst["dq"] <= 2e-2 and worst["dkv"] <= 2e-2, worst
+
+
+def test_config5_one_head_blocks_round_trip(gpu):
+    """The config 5 tensor moved as one-head blocks (head block size 1: 16384 blocks of 128 KiB, ragged):
+    gather through a seeded permutation, inverse scatter, bit for bit."""
+    from dcp_amd.ops.fused_ops import fused_copy_bf16_varlen
+
+    tokens, heads, d, bs = 262144, 32, 128, 512
+    n_blocks, numel = tokens // bs * heads, bs * d
+    rng = np.random.default_rng(1)
+    perm = rng.permutation(n_blocks)
+    n_tok = rng.integers(1, bs + 1, n_blocks)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    src = torch.randn(n_blocks, bs, d, device="cuda", generator=g).to(torch.bfloat16)  # [head block x block][token][d]
+    packed, back = torch.full_like(src, 7.0), torch.zeros_like(src)
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    i32 = lambda v: torch.tensor(np.ascontiguousarray(v), dtype=torch.int32, device="cuda")
+    ident, stride, n_el = np.arange(n_blocks), i32([numel] * n_blocks), i32(n_tok * d)
+    fused_copy_bf16_varlen(i64([src.data_ptr()] * n_blocks), i32(ident), stride, i64([packed.data_ptr()] * n_blocks),
+                           i32(perm), stride, n_el, numel, 128)
+    fused_copy_bf16_varlen(i64([packed.data_ptr()] * n_blocks), i32(perm), stride, i64([back.data_ptr()] * n_blocks),
+                           i32(ident), stride, n_el, numel, 128)
+    torch.cuda.synchronize()
+    valid = torch.arange(bs, device="cuda")[None, :] < torch.tensor(n_tok, device="cuda")[:, None]
+    s3, b3 = src.view(torch.int16), back.view(torch.int16)
+    assert torch.equal(b3[valid], s3[valid]) and bool((b3[~valid] == 0).all())
+    assert torch.equal(packed.view(torch.int16)[torch.tensor(perm, device="cuda")][valid], s3[valid])
 
 
 def test_config5_block_movement_full_size(gpu):
