@@ -173,7 +173,7 @@ _PROBES = None
 
 
 def load_probes():
-    """libbench_probes.so (bench_probes.hip, built by `python -m dcp_amd.build`): the two
+    """libbench_probes.so (bench_probes.hip, built by `python -m dcp_amd.build`): the
     measurement-only kernels this benchmark runs beside the product library."""
     global _PROBES
     if _PROBES is None:
@@ -187,6 +187,7 @@ def load_probes():
         lib = ctypes.CDLL(path)
         P, I = ctypes.c_void_p, ctypes.c_int
         lib.bench_mfma_probe.argtypes = [P, P, I, I, I, P, P]
+        lib.bench_mfma_mix_probe.argtypes = [P, P, I, I, I, P, P]
         lib.bench_hbm_stream_probe.argtypes = [P, P, I, ctypes.c_size_t, P]
         lib.bench_probe_last_error.restype = ctypes.c_char_p
         _PROBES = lib
@@ -232,6 +233,35 @@ def mfma_sustained(iters=60000):
         clocks, ticks = out[:2].tolist()
         res[name] = dict(TFLOPs=round(flop.value / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1),
                          shader_MHz=round(clocks / ticks * 100.0))
+    return res
+
+
+def mfma_with_instruction_mix(iters=4000):
+    """The MFMA probe again, two waves per SIMD and random operands, with every wave also issuing
+    what an attention kernel issues beside its MFMAs (vector instructions, exponentials, LDS
+    reads in the kernel's own proportions), evenly spread and free of dependencies, tile loads
+    and barriers: what no schedule of that instruction mix can exceed on this device."""
+    import ctypes
+
+    import torch
+
+    n_wg = 2 * torch.cuda.get_device_properties(0).multi_processor_count
+    n_words = n_wg * 256 * 16 * 8
+    g = torch.Generator(device="cuda").manual_seed(0)
+    ops = torch.randn(n_words, device="cuda", generator=g).to(torch.bfloat16)
+    out = torch.empty(2 + n_wg * 256, device="cuda", dtype=torch.float32)
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {}
+    for mix, name in enumerate(("attn_fwd_kernel", "attn_bwd_dkv_kernel", "attn_bwd_dq_kernel")):
+        flop = ctypes.c_double()
+        args = (ops.data_ptr(), out.data_ptr(), n_wg, iters, mix, ctypes.byref(flop), stream)
+        call_probe("bench_mfma_mix_probe", *args)  # warm-up
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        call_probe("bench_mfma_mix_probe", *args)
+        e1.record()
+        torch.cuda.synchronize()
+        res[name] = round(flop.value / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
     return res
 
 
@@ -609,6 +639,13 @@ def main():
         kernel_ms_per_step={k: round(v["ms_per_step"], 4) for k, v in sorted(kt.items())},
         mfma_only_kernel=mfma_sustained(),
     )
+    # executed MFMA rate of each attention kernel against what MFMAs sustain beside that kernel's
+    # own mix of other instructions (dependency-free, no loads, no barriers)
+    mix = mfma_with_instruction_mix()
+    executed = dict(attn_fwd_kernel=fwd_tflops, attn_bwd_dkv_kernel=extra["attn_bwd_dkv_kernel"]["executed_TFLOPs"],
+                    attn_bwd_dq_kernel=extra["attn_bwd_dq_kernel"]["executed_TFLOPs"])
+    extra["mfma_with_kernel_instruction_mix"] = {
+        k: dict(bound_TFLOPs=v, kernel_executed_frac_of_bound=round(executed[k] / v, 3)) for k, v in mix.items()}
     if not args.no_movement:
         del ex_f, ex_b
         torch.cuda.empty_cache()

@@ -1,6 +1,7 @@
-// libbench_probes.so: two measurement-only kernels that bench.py runs beside the product library
+// libbench_probes.so: three measurement-only kernels that bench.py runs beside the product library
 // for the roofline discussion (not part of libdcp_hip.so or of its C ABI; nothing in the
-// reference corresponds to them): the sustained matrix-core rate and the streaming rate of HBM.
+// reference corresponds to them): the sustained matrix-core rate, the same with an attention kernel's instruction mix beside the
+// MFMAs, and the streaming rate of HBM.
 // Built by `python -m dcp_amd.build` from this one file; entry points return 0 or a DCP_ERR_*
 // code and bench_probe_last_error() gives the message.
 //
@@ -61,6 +62,70 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const u32x
     out[0] = (float)(c1 - c0);
     out[1] = (float)(w1 - w0);
   }
+}
+
+// What the matrix cores sustain when every wave also issues, evenly spread between its MFMAs and
+// with no dependency on anything loaded, the other instructions an attention kernel needs per
+// NM MFMAs: NV plain vector instructions (FMAs), NE exponentials, NB128 16-byte and NB64 8-byte LDS
+// reads per lane.  Two workgroups per CU (64 KiB of LDS each), i.e. two waves per SIMD, like the
+// attention kernels.  No tile loads, no barriers, no waits on data: an upper bound for a kernel
+// with that instruction mix, whatever its schedule.
+template <int NM, int NV, int NE, int NB128, int NB64>
+__global__ __launch_bounds__(kProbeThreads, 2) void mfma_mix_probe_kernel(const u32x4* operands, float* out, int iters,
+                                                                         float s, float t) {
+  __shared__ __attribute__((aligned(16))) u32x4 lds[4096];  // 64 KiB: two workgroups per CU
+  for (int i = threadIdx.x; i < 4096; i += kProbeThreads) lds[i] = operands[i];
+  __syncthreads();
+  const size_t base = ((size_t)blockIdx.x * kProbeThreads + threadIdx.x) * 16;
+  const u32x4 a = operands[base], b = operands[base + 8];
+  f32x16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
+  float x[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) x[i] = threadIdx.x * 0.001f + i * 0.01f;
+  const uint32_t at = lds_address(&lds[0]) + (threadIdx.x & 63) * 16;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      acc[m & 3] = mfma_32x32x16<DCP_DTYPE_BF16>(a, b, acc[m & 3]);
+      // the m-th share of each kind: floor((m + 1) N / NM) - floor(m N / NM) instructions
+#pragma unroll
+      for (int k = m * NV / NM; k < (m + 1) * NV / NM; ++k) x[k & 15] = __builtin_fmaf(x[k & 15], s, t);
+#pragma unroll
+      for (int k = m * NE / NM; k < (m + 1) * NE / NM; ++k) x[k & 15] = fast_exp2(x[k & 15]);
+#pragma unroll
+      for (int k = m * NB128 / NM; k < (m + 1) * NB128 / NM; ++k) {
+        u32x4 v;
+        asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(v) : "v"(at));
+        asm volatile("" ::"v"(v));
+      }
+#pragma unroll
+      for (int k = m * NB64 / NM; k < (m + 1) * NB64 / NM; ++k) {
+        u32x2 v;
+        asm volatile("ds_read_b64 %0, %1 offset:2048" : "=v"(v) : "v"(at));
+        asm volatile("" ::"v"(v));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)");
+    if ((it & 63) == 63) {  // keep the sums finite
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[j][i] *= 1e-6f;
+    }
+  }
+  float r = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) r += acc[j][i];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r += x[i];
+  out[2 + (size_t)blockIdx.x * kProbeThreads + threadIdx.x] = r;
 }
 
 // Plain streaming kernel for the HBM roofline discussion: NS equally long input streams are
@@ -139,4 +204,34 @@ extern "C" int bench_mfma_probe(const void* operands, float* out, int n_workgrou
     hipLaunchKernelGGL(mfma_probe_kernel<DCP_DTYPE_FP16>, grid, block, 0, (hipStream_t)stream,
                        (const u32x4*)operands, out, iters);
   return check_launch("mfma_probe_kernel");
+}
+
+
+// The MFMA probe with an attention kernel's other instructions beside the MFMAs (see
+// mfma_mix_probe_kernel): `mix` 0 = forward (per 32 MFMAs: 112 FMAs, 32 exponentials, 16 + 32 LDS
+// reads), 1 = dK/dV kernel (per 32: 58, 16, 20 + 32), 2 = dQ kernel (per 48: 80, 32, 32 + 32).
+// `n_workgroups` workgroups of 256 threads, two per CU; `operands` and `out` as for
+// bench_mfma_probe (at least 4096 x 16 bytes of operands).  *flop = the MFMAs' operations.
+extern "C" int bench_mfma_mix_probe(const void* operands, float* out, int n_workgroups, int iters, int mix, double* flop,
+                                    void* stream) {
+  DCP_REQUIRE(operands && out && flop, "mfma_mix_probe: null argument");
+  DCP_REQUIRE(n_workgroups >= 16 && iters > 0, "mfma_mix_probe: at least 16 workgroups and one iteration");
+  const int per_iter = mix == 2 ? 48 : 32;
+  *flop = (double)n_workgroups * (kProbeThreads / 64) * (double)iters * per_iter * (2.0 * 32 * 32 * 16);
+  dim3 grid(n_workgroups), block(kProbeThreads);
+  const u32x4* ops = (const u32x4*)operands;
+  switch (mix) {
+    case 0:
+      hipLaunchKernelGGL((mfma_mix_probe_kernel<32, 112, 32, 16, 32>), grid, block, 0, (hipStream_t)stream, ops, out, iters, 1.0001f, 0.5f);
+      break;
+    case 1:
+      hipLaunchKernelGGL((mfma_mix_probe_kernel<32, 58, 16, 20, 32>), grid, block, 0, (hipStream_t)stream, ops, out, iters, 1.0001f, 0.5f);
+      break;
+    case 2:
+      hipLaunchKernelGGL((mfma_mix_probe_kernel<48, 80, 32, 32, 32>), grid, block, 0, (hipStream_t)stream, ops, out, iters, 1.0001f, 0.5f);
+      break;
+    default:
+      return fail(DCP_ERR_UNSUPPORTED, "mfma_mix_probe: mix %d unsupported (0, 1 or 2)", mix);
+  }
+  return check_launch("mfma_mix_probe_kernel");
 }
