@@ -202,3 +202,38 @@ def test_config1_fp32_merge_of_up_to_eight_partials(gpu):
     torch.cuda.synchronize()
     assert max_abs_err(dst_out.cpu().numpy(), t_out) <= 1e-5
     assert max_abs_err(dst_lse.cpu().numpy(), t_lse) <= 1e-5
+
+
+@pytest.mark.parametrize("seed,d,bs,hq,hkv", [(21, 128, 128, 4, 2), (22, 64, 64, 2, 2), (23, 128, 64, 8, 2)])
+def test_arbitrary_ranges(gpu, seed, d, bs, hq, hkv):
+    """Ranges no mask generator produces: starts and ends anywhere (inside tiles, past the row's
+    keys, below zero length), empty ranges beside full ones, two ranges that overlap, touch or
+    nest, queries that attend a single key, rows whose queries do not fill the block.  The
+    kernels classify tiles from the hull and the core of a tile's ranges and mask the rest bit by
+    bit, so every row mixes skipped, unmasked and masked tiles."""
+    rng = np.random.default_rng(seed)
+    rows = []
+    for _ in range(6):
+        nblk = int(rng.integers(1, 6))
+        nq = int(rng.choice([bs, bs, int(rng.integers(1, bs + 1))]))
+        n_keys = nblk * bs
+        n_ranges = int(rng.integers(1, 3))
+        ranges = np.zeros((n_ranges, 2, nq), dtype=np.int64)
+        for r in range(n_ranges):
+            kind = rng.integers(0, 5, size=nq)
+            s = rng.integers(0, n_keys + 1, size=nq)
+            e = rng.integers(0, n_keys + bs, size=nq)            # may lie past the row's keys, or before the start
+            s = np.where(kind == 0, 0, s)                         # from the first key
+            e = np.where(kind == 1, s + 1, e)                     # a single key (or none, at the very end)
+            e = np.where(kind == 2, s, e)                         # empty
+            s, e = np.where(kind == 3, 0, s), np.where(kind == 3, n_keys, e)  # everything
+            if r == 0 and rng.integers(0, 2):                     # a smooth band, so that whole tiles are unmasked
+                t = np.arange(nq)
+                s, e = np.maximum(t * n_keys // max(nq, 1) - bs, 0), np.minimum(t * n_keys // max(nq, 1) + bs + 1, n_keys)
+            ranges[r, 0], ranges[r, 1] = s, e
+        rows.append((nq, nblk, ranges))
+    pr = _paged_rows(gpu, rows, bs, hq=hq, hkv=hkv, d=d, seed=seed)
+    with np.errstate(invalid="ignore"):  # queries that attend nothing: +inf against +inf
+        worst = _check_direct(pr, _run_direct(pr))
+    assert worst["out"] <= OUT_TOL and worst["dq"] <= GRAD_TOL and worst["dkv"] <= GRAD_TOL, worst
+    assert not worst["lse"] > LSE_TOL, worst
