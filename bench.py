@@ -466,23 +466,24 @@ def exchange_microbench(n_devices=4, blocks_per_pair=64, bs=1024, hb=4, d=128, i
 
 
 # ---------------------------------------------------------------------------
-# CPU baseline: the oracle on a bounded, seeded sample of q-block rows
+# CPU baseline: dense masked attention in torch on a bounded, seeded sample of q-block rows
 # ---------------------------------------------------------------------------
 
 
 def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
-    """Times the numpy oracle's fwd+bwd of whole q-block rows (all heads of the
-    row's head block) drawn from the workload's backward plan until about
-    ``budget_s`` seconds of CPU work are done."""
+    """Times dense masked attention, forward and backward, of whole q-block rows (all heads of the
+    row's head block against the row's keys) drawn from the workload's plan, in fp32 torch on the
+    host cores (oracle/torch_cpu_path.py: the form of the reference's own dense check, the only
+    CPU-expressible statement of this path it holds), until about ``budget_s`` seconds of CPU
+    work are done.  One untimed row first."""
+    import torch
+
     from oracle import dcp_oracle as oracle
+    from oracle.torch_cpu_path import row_attention_fwd_bwd
 
-    # the threads the oracle's matrix products really run on (numpy's BLAS pool); no silent default
-    from threadpoolctl import threadpool_info
-
-    pools = [p["num_threads"] for p in threadpool_info() if p.get("user_api") == "blas"]
-    if not pools:
-        raise SystemExit("bench.py: cannot tell how many threads numpy's BLAS uses (no BLAS pool reported by threadpoolctl)")
-    threads = max(pools)
+    threads = torch.get_num_threads()  # the intra-op pool torch's CPU kernels run on (OMP_NUM_THREADS honoured)
+    if not threads or threads < 1:
+        raise SystemExit("bench.py: torch reports no CPU threads")
     instr = next(i for i in fw.instructions if type(i).__name__ == "AttnInstr")
     mask = np.asarray(instr.attn_mask)
     if mask.ndim == 2:
@@ -493,16 +494,15 @@ def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
     hkv = max(1, hb // (wl["n_heads"] // wl["n_groups"]))
     cu = np.concatenate(([0], np.cumsum(instr.seqlens_q)))
     pairs, rows, elapsed = 0, 0, 0.0
-    for b in order:
+    f32 = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32))
+    for n, b in enumerate([order[0]] + list(order)):
         n_kv = instr.seqlens_kv[b]
-        q = (rng.standard_normal((bs, hb, d)) * 0.5).astype(np.float32)
-        k = (rng.standard_normal((n_kv, hkv, d)) * 0.5).astype(np.float32)
-        v = (rng.standard_normal((n_kv, hkv, d)) * 0.5).astype(np.float32)
-        dout = rng.standard_normal((bs, hb, d)).astype(np.float32)
-        allowed = oracle.ranges_to_bool(mask[:, :, cu[b] : cu[b + 1]], n_kv)
+        q, k, v, dout = f32(bs, hb, d) * 0.5, f32(n_kv, hkv, d) * 0.5, f32(n_kv, hkv, d) * 0.5, f32(bs, hb, d)
+        allowed = torch.from_numpy(oracle.ranges_to_bool(mask[:, :, cu[b] : cu[b + 1]], n_kv))
         t0 = time.perf_counter()
-        out, lse = oracle.range_attention_fwd(q, k, v, allowed, dtype=np.float32)
-        oracle.range_attention_bwd(q, k, v, out, lse, dout, allowed, dtype=np.float32)
+        row_attention_fwd_bwd(q, k, v, dout, allowed)
+        if n == 0:
+            continue  # warm-up
         elapsed += time.perf_counter() - t0
         pairs += int(allowed.sum())
         rows += 1
@@ -511,7 +511,8 @@ def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
     flops = oracle.attention_flops(pairs, hb, d, "fwd+bwd")
     return dict(
         value=round(flops / elapsed / 1e12, 5), unit="TFLOP/s", cores=int(threads), kind="port",
-        sample=f"{rows} seeded q-block rows of the same schedule (fwd+bwd, fp32 numpy oracle, {elapsed:.1f} s)",
+        sample=f"{rows} seeded q-block rows of the same schedule (fwd+bwd, dense masked attention in fp32 torch on the host, "
+               f"{elapsed:.1f} s)",
     )
 
 

@@ -226,3 +226,27 @@ def test_flop_convention():
     assert oracle.attention_flops(10, 2, 8, "fwd") == 4 * 10 * 2 * 8
     assert oracle.attention_flops(10, 2, 8, "bwd") == 2.5 * 4 * 10 * 2 * 8
     assert oracle.attention_flops(10, 2, 8, "fwd+bwd") == 14 * 10 * 2 * 8
+
+
+def test_torch_cpu_row_path_equals_the_numpy_oracle():
+    """bench.py's CPU baseline (oracle/torch_cpu_path.py, fp32 torch on the host) against the numpy
+    oracle in fp64: GQA, two ranges, a query that attends nothing."""
+    from oracle.torch_cpu_path import row_attention_fwd_bwd
+
+    rng = np.random.default_rng(9)
+    Tq, Tk, H, Hkv, D = 37, 90, 4, 2, 32
+    q, dout = rng.standard_normal((Tq, H, D)), rng.standard_normal((Tq, H, D))
+    k, v = rng.standard_normal((Tk, Hkv, D)), rng.standard_normal((Tk, Hkv, D))
+    t = np.arange(Tq)
+    ranges = np.stack([np.stack([t * 0, np.minimum(t, 5)]), np.stack([t + 20, t + 41])])
+    ranges[:, :, 11] = 0  # query 11 attends nothing (query 0's first range is empty too)
+    allowed = oracle.ranges_to_bool(ranges, Tk)
+    w_out, w_lse = oracle.range_attention_fwd(q, k, v, allowed)
+    w_dq, w_dk, w_dv = oracle.range_attention_bwd(q, k, v, w_out, w_lse, dout, allowed)
+    f32 = lambda x: torch.from_numpy(np.asarray(x, dtype=np.float32))
+    out, lse, dq, dk, dv = row_attention_fwd_bwd(f32(q), f32(k), f32(v), f32(dout), torch.from_numpy(allowed))
+    assert np.isposinf(lse.numpy()[:, 11]).all() and np.isposinf(w_lse[:, 11]).all()
+    fin = np.isfinite(w_lse)
+    assert np.abs(lse.numpy()[fin] - w_lse[fin]).max() <= 1e-5
+    for got, want in ((out, w_out), (dq, w_dq), (dk, w_dk), (dv, w_dv)):
+        assert np.abs(got.numpy() - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
