@@ -298,20 +298,37 @@ class DCPAttention(torch.autograd.Function):
 # ---------------------------------------------------------------------------
 
 
+def _size_classes(block_numels) -> dict:
+    """``{block numel: class}`` such that blocks within a factor of four of a class's largest share
+    a launch: its grid is sized for the largest of them, so at most three in four workgroups of
+    the smallest find nothing to do, whereas a 64 KiB block in a grid sized for 4 MiB blocks would
+    idle 63 in 64.  (Q and KV blocks of one plan, a factor 2 to 5 apart at most head layouts, land
+    in one class.)"""
+    classes, top = {}, None
+    for n in sorted(set(int(x) for x in block_numels), reverse=True):
+        if top is None or n * 4 < top:
+            top = n
+        classes[n] = top
+    return classes
+
+
 def _prepare_memcpy(exec: AttentionExecutor, instr: MemcpyInstr):
-    """One argument table per dtype for data blocks and one for LSE blocks.  The source is the
-    unpadded buffer, addressed by ``local_cu_seqlens`` (reference ``_prepare_memcpy`` :606-790,
-    which makes one table, and one launch, per (dtype, block numel): here blocks of different
+    """One argument table per (dtype, size class) for data blocks and one for LSE blocks.  The source
+    is the unpadded buffer, addressed by ``local_cu_seqlens`` (reference ``_prepare_memcpy`` :606-790,
+    which makes one table, and one launch, per (dtype, block numel): here blocks of similar
     sizes share a launch, whose grid is sized for the largest -- every block carries its own
     element count and stride, and the workgroups past a smaller block's end leave at once)."""
     cu = exec.execution_plan.local_cu_seqlens
     data = defaultdict(lambda: [[] for _ in range(7)])
     lse = defaultdict(lambda: [[] for _ in range(7)])
     head_block_size = None
+    size_class = _size_classes(exec.buffer_block_strides[src.buffer_type] for src, _ in instr.src_dst_pairs
+                               if src.buffer_type not in _LSE_BUFFER_TYPES)
     for src, dst in instr.src_dst_pairs:
         src_buf, dst_buf = exec.buffers[src.buffer_type], exec.buffers[dst.buffer_type]
         src_off = cu[src.index]
-        key = (src_buf.dtype, exec.buffer_block_strides[src.buffer_type]) if src.buffer_type in _LSE_BUFFER_TYPES else src_buf.dtype
+        key = ((src_buf.dtype, exec.buffer_block_strides[src.buffer_type]) if src.buffer_type in _LSE_BUFFER_TYPES
+               else (src_buf.dtype, size_class[exec.buffer_block_strides[src.buffer_type]]))
         if src.buffer_type in _LSE_BUFFER_TYPES:
             assert dst.buffer_type in _LSE_BUFFER_TYPES
             cols = lse[key]
@@ -346,7 +363,7 @@ def _prepare_memcpy(exec: AttentionExecutor, instr: MemcpyInstr):
 
     exec._args_cache[exec.instr_index] = {
         # key: (dtype, the largest block numel of the launch)
-        "other": {(dtype, max(cols[5])): tables(cols) for dtype, cols in data.items()},
+        "other": {(dtype, max(cols[5])): tables(cols) for (dtype, _), cols in data.items()},
         "lse": {key: tables(cols) + (head_block_size,) for key, cols in lse.items()},
     }
 
@@ -585,12 +602,13 @@ def _handle_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
 def _prepare_sum(exec: AttentionExecutor, instr: SumInstr):
     groups = defaultdict(lambda: defaultdict(list))
     cu = exec.execution_plan.local_cu_seqlens
-    # one launch per dtype: sums over blocks of different sizes share it (its grid is sized for the
-    # largest block, every sum carries its own element count and strides)
+    # one launch per (dtype, size class): sums over blocks of similar sizes share it (its grid is
+    # sized for the largest block, every sum carries its own element count and strides)
+    size_class = _size_classes(exec.buffer_block_strides[op.src_buffers[0].buffer_type] for op in instr.ops)
     for op in instr.ops:
         src_type = op.src_buffers[0].buffer_type
         dst_type = op.dst_buffer.buffer_type
-        g = groups[exec.buffers[src_type].dtype]
+        g = groups[(exec.buffers[src_type].dtype, size_class[exec.buffer_block_strides[src_type]])]
         per_token = int(np.prod(exec.buffer_per_token_shape[src_type]))
         g["src_ptrs"].append(exec.buffers[src_type].data_ptr())
         g["src_offsets"].append([blk.index for blk in op.src_buffers])
@@ -605,7 +623,7 @@ def _prepare_sum(exec: AttentionExecutor, instr: SumInstr):
             g["dst_strides"].append(exec.buffer_block_strides[dst_type])
         g["n_elems"].append(op.dst_buffer.n_tokens * per_token)
     prepared = {}
-    for dtype, g in groups.items():
+    for (dtype, _), g in groups.items():
         width = _round_to_pow_2(max(g["n_ops"]))
         padded = [row + [-1] * (width - len(row)) for row in g["src_offsets"]]
         prepared[(dtype, max(g["src_strides"]))] = (

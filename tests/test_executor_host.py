@@ -84,3 +84,14 @@ def test_attention_wrappers_reject_block_tables_of_the_wrong_shape():
         _check_tables(3, i32(5), None, ok, dict(kv_block_table=i32(3, 5)))
     with pytest.raises(ValueError, match="row_order"):
         _check_tables(3, i32(4), i32(2), ok, dict(kv_block_table=i32(3, 5)))
+
+
+def test_blocks_share_a_launch_only_within_a_factor_of_four():
+    from dcp_amd.runtime.flash_attention.executor import _size_classes
+
+    c = _size_classes([524288, 262144, 327680, 131072, 131071, 4096, 1 << 22, 65536, 16385])
+    assert c[524288] == c[262144] == c[327680] == c[131072] == 524288  # Q and KV blocks of one plan
+    assert c[131071] == 131071 and c[65536] == 131071  # just under a quarter of the largest: the next class starts
+    assert c[1 << 22] == 1 << 22 and c[4096] == 4096 and c[16385] == 16385
+    for n, top in c.items():
+        assert n <= top <= 4 * n
