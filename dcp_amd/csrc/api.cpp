@@ -21,6 +21,8 @@ struct Span {
 std::mutex g_mu;
 bool g_profiling = false;
 std::vector<Span> g_spans;
+unsigned g_generation = 0;  // bumped whenever a report clears the list: span ids carry it
+constexpr int kSpanBits = 24;
 }  // namespace
 
 bool profiling_enabled() { return g_profiling; }
@@ -35,15 +37,23 @@ int profile_begin(const char* name, hipStream_t stream) {
     return -1;
   }
   (void)hipEventRecord(s.start, stream);
+  if (g_spans.size() >= (size_t)1 << kSpanBits) {  // ids are 24 bits of index under 7 bits of generation
+    (void)hipEventDestroy(s.start);
+    (void)hipEventDestroy(s.stop);
+    return -1;
+  }
   g_spans.push_back(s);
-  return (int)g_spans.size() - 1;
+  return (int)(((g_generation & 0x7f) << kSpanBits) | (unsigned)(g_spans.size() - 1));
 }
 
 void profile_end(int span, hipStream_t stream) {
   std::lock_guard<std::mutex> lock(g_mu);
-  // the span this timer opened (none if its events could not be created, or if a report has
-  // cleared the list in between)
-  if (span >= 0 && span < (int)g_spans.size()) (void)hipEventRecord(g_spans[span].stop, stream);
+  // The span this timer opened: none if its events could not be created, and none if a report
+  // has cleared the list in between (the id's generation then differs, and the index may by now
+  // name another kernel's span, whose stop event must not be recorded here).
+  if (span < 0 || (unsigned)(span >> kSpanBits) != (g_generation & 0x7f)) return;
+  const int index = span & ((1 << kSpanBits) - 1);
+  if (index < (int)g_spans.size()) (void)hipEventRecord(g_spans[index].stop, stream);
 }
 
 }  // namespace dcp
@@ -71,6 +81,7 @@ extern "C" int dcp_profile_report(char* buffer, size_t capacity) {
     (void)hipEventDestroy(s.stop);
   }
   dcp::g_spans.clear();
+  ++dcp::g_generation;
   std::string text;
   char line[256];
   for (auto& kv : totals) {

@@ -994,7 +994,13 @@ void* scratch_on_current_device() {
 }
 }  // namespace
 
-extern "C" size_t dcp_attn_bwd_static_scratch_bytes(void) { return DCP_ATTN_BWD_STATIC_SCRATCH_BYTES; }
+// Also the set-up call of dcp_attn_bwd_static: it looks up (and keeps) the scratch array's address
+// on the current device, so that the entry point itself makes no runtime query -- a caller that
+// records it into a HIP graph calls this once per device beforehand, outside the capture.
+extern "C" size_t dcp_attn_bwd_static_scratch_bytes(void) {
+  (void)scratch_on_current_device();
+  return DCP_ATTN_BWD_STATIC_SCRATCH_BYTES;
+}
 
 extern "C" int dcp_attn_bwd_static(const void* dout, const void* q, const void* k, const void* v,
                                    const void* out, const float* lse, void* dq, void* dk, void* dv,

@@ -42,6 +42,9 @@ __device__ __forceinline__ u32x4 pack_vec16(const float (&acc)[Vec16<DTYPE>::N])
   return bits;
 }
 
+// Only the two infinities mark an empty source (the reference tests lse != -inf and lse != inf):
+// a NaN LSE takes part in the merge and makes the merged LSE and output of its (token, head) NaN.
+// fmaxf drops a NaN operand, so the kernels note one and put it into the running maximum themselves.
 __device__ __forceinline__ bool lse_is_finite(float l) {
   return l != INFINITY && l != -INFINITY;
 }
@@ -157,11 +160,14 @@ __global__ __launch_bounds__(kMergeThreads) void merge_out_lse_kernel(
 #pragma unroll
       for (int k = 0; k < TPG; ++k) {
         float m_new = m[k];
+        bool nan_seen = false;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           if (j0 + u >= n_src || !lse_is_finite(l[k][u])) l[k][u] = -INFINITY;
           m_new = fmaxf(m_new, l[k][u]);
+          nan_seen |= l[k][u] != l[k][u];
         }
+        if (nan_seen) m_new = NAN;  // sums and weights below turn NaN and stay so
         if (m_new == -INFINITY) continue;  // nothing finite so far
         const float rescale = expf(m[k] - m_new);  // m = -inf -> 0
         ssum[k] *= rescale;
@@ -274,12 +280,15 @@ __global__ __launch_bounds__(kMergeThreads) void merge_rows_kernel(
     if (t0 + t >= n_tok) continue;
     const float* lse_row = src_lse + (int64_t)h * src_lse_head_stride + t0 + t;
     float m = -INFINITY;
+    bool nan_seen = false;
     for (int j = 0; j < n_src; ++j) {
       float l = lse_row[(int64_t)slot[j] * lse_block_stride];
       if (!lse_is_finite(l)) l = -INFINITY;
       weight[j * plane + pair] = l;
       m = fmaxf(m, l);
+      nan_seen |= l != l;
     }
+    if (nan_seen) m = NAN;  // the sum, the merged LSE and every weight of a non-empty source turn NaN
     float new_lse = -1.0f;
     if (m != -INFINITY) {
       float ssum = 0.0f;

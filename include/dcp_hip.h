@@ -261,9 +261,13 @@ size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
  * forbid hipMalloc).  No counterpart in the reference.  Same arguments, results
  * and errors as dcp_attn_bwd without `workspace`/`workspace_bytes`: the scratch
  * is a static device array inside the library, DCP_ATTN_BWD_STATIC_SCRATCH_BYTES
- * long, which every GPU the library runs on holds until the process ends (its
- * address is looked up at the first call on a device).  The call allocates and
- * frees nothing.  Sizes for which dcp_attn_bwd_workspace_bytes(...) exceeds the
+ * long, which every GPU the library runs on holds until the process ends.  Its
+ * address on a device is looked up once, by the first of
+ * dcp_attn_bwd_static_scratch_bytes() or dcp_attn_bwd_static() called with that
+ * device current: a caller that records dcp_attn_bwd_static into a HIP graph
+ * calls dcp_attn_bwd_static_scratch_bytes() once per device beforehand, outside
+ * the capture, and the recorded call then makes no runtime query.  The call
+ * allocates and frees nothing.  Sizes for which dcp_attn_bwd_workspace_bytes(...) exceeds the
  * scratch are rejected with DCP_ERR_ARG.  All calls on one GPU share the one
  * array: calls that may overlap on that GPU (different streams, or graphs
  * replayed side by side) race; calls that follow each other on a stream do not.

@@ -95,11 +95,13 @@ def block_copy(src_flat, src_elem_offsets, dst_flat, dst_elem_offsets, n_element
 def merge_out_lse(outs: np.ndarray, lses: np.ndarray):
     """outs [S, T, H, D], lses [S, H, T] -> (out [T, H, D], lse [H, T]).
 
-    Sources with lse = +-inf are ignored; with no finite source lse = -1 and
-    out = 0 (fused_ops.py:118-143)."""
+    Sources with lse = +-inf are ignored; with no other source lse = -1 and
+    out = 0 (fused_ops.py:118-143).  Only the two infinities mark an empty source
+    (fused_ops.py:123: ``lse != -inf and lse != inf``): a NaN lse counts as a source and
+    makes the merged lse and out of its (token, head) NaN."""
     outs = np.asarray(outs, dtype=np.float64)
     lses = np.asarray(lses, dtype=np.float64)
-    finite = np.isfinite(lses)
+    finite = ~np.isinf(lses)
     masked = np.where(finite, lses, NEG_INF)
     m = masked.max(axis=0)
     any_finite = finite.any(axis=0)

@@ -116,7 +116,65 @@ def run_executor(case, backward=False, use_graph=False, synchronous=False, poiso
     return res, ex
 
 
-def run_plan_oracle(case, backward=False):
+def storage_ulp(x, dtype="bf16"):
+    """Spacing of the 16-bit storage type at |x| (bf16: 8 significand bits, fp16: 11)."""
+    x = np.maximum(np.abs(np.asarray(x, dtype=np.float64)), 2.0 ** -126 if dtype == "bf16" else 2.0 ** -14)
+    return 2.0 ** (np.floor(np.log2(x)) - (7 if dtype == "bf16" else 10))
+
+
+class SlackPlanOracle(oracle.PlanOracle):
+    """The plan interpreter, which also keeps for every element of the 16-bit buffers how far a second
+    exact run of the same plan may end up from this one through rounding alone: wherever the plan
+    stores a value in 16 bits, a difference in the last bits of the value before rounding can move
+    the stored value by one step of the type AT THAT VALUE's magnitude; a sum passes its sources'
+    steps on and adds its own, a merge (a convex combination) passes on the largest.  This is what
+    makes a bound of "a few steps of the result" wrong for a dK that is the small sum of large
+    replicas, and it is all the slack a comparison of the kernels with the interpreter needs
+    beyond the kernels' own arithmetic."""
+
+    def __init__(self, plan, hb, head_dim, dtype="bf16"):
+        super().__init__(plan, hb, head_dim)
+        self.dtype = dtype
+        self.slack = {name: np.zeros(buf.shape) for name, buf in self.buffers.items()
+                      if self.store_dtype[name] != "fp32"}
+        self._carried = 0.0
+
+    def _store(self, name, index, value):
+        super()._store(name, index, value)
+        if name in self.slack:
+            # (the step just above the value: the other run may land across a power of two)
+            self.slack[name][index] = self._carried + storage_ulp(1.01 * self.buffers[name][index], self.dtype)
+
+    def _MemcpyInstr(self, instr):
+        super()._MemcpyInstr(instr)
+        cu = self.plan.local_cu_seqlens
+        for src, dst in instr.src_dst_pairs:
+            if dst.buffer_type in self.slack and src.buffer_type in self.slack:
+                off = cu[src.index]
+                self.slack[dst.buffer_type][dst.index, : src.n_tokens] = self.slack[src.buffer_type][off : off + src.n_tokens]
+
+    def _AttnReductionInstr(self, instr):
+        for op in instr.ops:
+            n = op.dst_buffer[0].n_tokens
+            self._carried = np.max([self.slack[o.buffer_type][o.index, :n] for o, _ in op.src_buffers], axis=0)
+            super()._AttnReductionInstr(type("One", (), dict(ops=[op], output_is_unpadded=instr.output_is_unpadded))())
+        self._carried = 0.0
+
+    def _SumInstr(self, instr):
+        for op in instr.ops:
+            n = op.dst_buffer.n_tokens
+            self._carried = np.sum([self.slack[s.buffer_type][s.index, :n] for s in op.src_buffers], axis=0)
+            if len(op.src_buffers) == 1:  # a copy rounds nothing
+                self._carried = self._carried - storage_ulp(1.01 * self.buffers[op.src_buffers[0].buffer_type][op.src_buffers[0].index, :n], self.dtype)
+            super()._SumInstr(type("One", (), dict(ops=[op], output_is_unpadded=instr.output_is_unpadded))())
+        self._carried = 0.0
+
+
+def run_plan_oracle(case, backward=False, with_slack=False):
+    """The plans on the oracle's interpreter; global-layout results like run_executor.  With
+    ``with_slack`` also the rounding slack of out, dq and dkv (see SlackPlanOracle), in the same layout."""
+    if with_slack:
+        return _run_plan_oracle_with_slack(case)
     layout = case["layout"]
     po = oracle.PlanOracle(case["fw"], case["head_block"], case["head_dim"])
     po.set("LocalQ", layout.to_local_q(case["q"]).float().numpy())
@@ -136,6 +194,31 @@ def run_plan_oracle(case, backward=False):
         res += [layout.from_local_q(torch.from_numpy(b2["LocaldQ"].copy())),
                 layout.from_local_kv(torch.from_numpy(b2["LocaldKV"].copy()))]
     return res
+
+
+def _run_plan_oracle_with_slack(case):
+    layout = case["layout"]
+    po = SlackPlanOracle(case["fw"], case["head_block"], case["head_dim"], case["dtype"])
+    po.set("LocalQ", layout.to_local_q(case["q"]).float().numpy())
+    po.set("LocalKV", layout.to_local_kv(case["kv"]).float().numpy())
+    po.slack["LocalQ"][...] = 0.0  # inputs are given, not computed
+    po.slack["LocalKV"][...] = 0.0
+    bufs = po.run()
+    pb = SlackPlanOracle(case["bw"], case["head_block"], case["head_dim"], case["dtype"])
+    pb.set("LocalQ", layout.to_local_q(case["q"]).float().numpy())
+    pb.set("LocalKV", layout.to_local_kv(case["kv"]).float().numpy())
+    pb.set("LocalOut", bufs["LocalOut"])
+    pb.buffers["LocalLSE"][...] = bufs["LocalLSE"]
+    pb.set("LocaldOut", layout.to_local_q(case["dout"]).float().numpy())
+    for name in ("LocalQ", "LocalKV", "LocalOut", "LocaldOut"):
+        pb.slack[name][...] = 0.0
+    b2 = pb.run()
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32))
+    res = [layout.from_local_q(t(bufs["LocalOut"])), layout.from_local_lse(t(bufs["LocalLSE"])),
+           layout.from_local_q(t(b2["LocaldQ"])), layout.from_local_kv(t(b2["LocaldKV"]))]
+    slack = [layout.from_local_q(t(po.slack["LocalOut"])), None, layout.from_local_q(t(pb.slack["LocaldQ"])),
+             layout.from_local_kv(t(pb.slack["LocaldKV"]))]
+    return res, slack
 
 
 # ---------------------------------------------------------------------------

@@ -91,6 +91,48 @@ def test_forward_matches_plan_oracle_buffers(gpu):
     assert np.abs(res[1].numpy() - ref[1].numpy()).max() <= LSE_TOL
 
 
+# Same plan, same storage roundings: the oracle's interpreter keeps every buffer in the plan's own
+# types (partial outputs, dQ versions and dK/dV replicas rounded to 16 bits where the plan stores
+# them), so what is left between the two is the kernels' arithmetic (fp32 accumulation, P and dS
+# rounded to 16 bits before the second products) and, wherever a value is stored, one step of the
+# type at that value when the two sides land on different sides of a tie.  The interpreter adds
+# those steps up per element along the plan (tests/plan_cases.py: SlackPlanOracle).  The bound is
+# one and a half times that sum (a stored value may land one step away, and the arithmetic error
+# that pushed it over the tie, below half a step of that value, travels on with it) plus, for the
+# arithmetic itself, 5e-3 on out and dQ and 1e-2 * max(1, |ref|) on dK/dV (sums over every query of
+# the row and every head of the group, where P and dS rounded to 16 bits add up): a quarter and a
+# half of the bounds against dense attention.  The bound against dense attention (2e-2) has no room for
+# the plan's own rounding in replica-heavy plans; this one does not need it.
+TIGHT_CASES = {
+    # one 65-token sequence, four one-head q head blocks per kv head, two partials per row: dK is the
+    # sum of four bf16 replicas of magnitude 2-4 that cancel to ~0.1 (0.025 off dense attention)
+    "replicas_cancel": dict(seqlens=[65], block_size=128, n_heads=16, n_groups=4, head_dim=128, head_block=1,
+                            n_kv_groups=2, qkv_scale=0.5, seed=2027),
+    "gqa_split3": dict(seqlens=[700, 130], block_size=128, n_heads=4, n_groups=2, head_dim=128, head_block=1,
+                       n_kv_groups=3, qkv_scale=0.5),
+    "folded_stages": dict(seqlens=[900, 260], block_size=128, n_heads=4, n_groups=2, head_dim=64, head_block=2,
+                          n_kv_groups=4, fold=True, qkv_scale=0.5),
+    "lambda_two_ranges": dict(seqlens=[600, 150], block_size=128, n_heads=4, n_groups=1, head_dim=128, head_block=4,
+                              mask="lambda", mask_kwargs=dict(n_starting=16, l_pretrain=200), n_kv_groups=2,
+                              qkv_scale=0.5),
+}
+
+
+@pytest.mark.parametrize("name", list(TIGHT_CASES))
+def test_backward_matches_plan_oracle_with_the_same_roundings(gpu, name):
+    case = make_case(**TIGHT_CASES[name])
+    res, _ = run_executor(case, backward=True)
+    ref, slack = run_plan_oracle(case, backward=True, with_slack=True)
+    for what, got, want, room in zip(("out", "lse", "dq", "dkv"), res, ref, slack):
+        got, want = got.float().numpy().astype(np.float64), want.float().numpy().astype(np.float64)
+        if what == "lse":
+            assert np.abs(got - want).max() <= LSE_TOL, what
+            continue
+        arithmetic = 1e-2 * np.maximum(1.0, np.abs(want)) if what == "dkv" else 5e-3
+        excess = np.abs(got - want) - (1.5 * room.numpy().astype(np.float64) + arithmetic)
+        assert excess.max() <= 0.0, (what, float(excess.max()), float(np.abs(got - want).max()))
+
+
 # Head sizes the kernels are not built for run zero-padded at the next one that is (64, 128), as
 # the reference pads head sizes to what its kernels take: multiples of 8 and one that is not.
 FWD_CASES.update({

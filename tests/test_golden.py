@@ -85,9 +85,9 @@ def test_hip_path_matches_golden_attention(gpu, name):
     case = dict(fw=fw, bw=bw, layout=layout, mask=mask, q=q, kv=kv, dout=dout, seqlens=seqlens,
                 head_block=head_block, head_dim=head_dim, dtype="bf16")
     (out, lse, dq, dkv), _ = run_executor(case, backward=True)
-    # outputs and LSE: max-abs 2e-2 / 1e-3; gradients: 2e-2 relative to max(1, |ref|)
+    # out and dQ: pure max-abs 2e-2; LSE 1e-3; dK/dV: 2e-2 relative to max(1, |ref|)
     assert np.abs(out.float().numpy() - z["out"]).max() <= 2e-2
     assert np.abs(lse.float().numpy() - z["lse"]).max() <= 1e-3
-    for got, key in ((dq, "dq"), (dkv, "dkv")):
-        ref = z[key]
-        assert (np.abs(got.float().numpy() - ref) <= 2e-2 * np.maximum(1.0, np.abs(ref))).all(), key
+    assert np.abs(dq.float().numpy() - z["dq"]).max() <= 2e-2
+    ref = z["dkv"]
+    assert (np.abs(dkv.float().numpy() - ref) <= 2e-2 * np.maximum(1.0, np.abs(ref))).all(), "dkv"

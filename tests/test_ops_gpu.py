@@ -118,7 +118,7 @@ def test_fused_copy_lse_bit_exact(gpu, heads):
 
 
 def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, inf_frac=0.0,
-                unpadded=True):
+                unpadded=True, nan_frac=0.0):
     from dcp_amd.ops.fused_ops import flash_attn_update_out_lse
 
     g = torch.Generator().manual_seed(seed)
@@ -133,6 +133,8 @@ def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, in
         u = torch.rand(src_lse.shape, generator=g)
         src_lse[u < inf_frac / 2] = float("inf")
         src_lse[(u >= inf_frac / 2) & (u < inf_frac)] = float("-inf")
+    if nan_frac > 0:
+        src_lse[torch.rand(src_lse.shape, generator=g) < nan_frac] = float("nan")
     blocks = rng.permutation(n_src_blocks)[: sum(n_src_per_op)]
     width = 1 << (max(n_src_per_op) - 1).bit_length()
     table, c = [], 0
@@ -173,8 +175,14 @@ def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, in
     max_out = max_lse = 0.0
     for op in range(n_ops):
         n, off = n_tokens[op], dst_offsets[op]
-        max_out = max(max_out, np.abs(got_out[off : off + n] - exp_out[op]).max())
-        max_lse = max(max_lse, np.abs(got_lse[:, off : off + n] - exp_lse[op]).max())
+        g_out, g_lse = got_out[off : off + n], got_lse[:, off : off + n]
+        if nan_frac > 0:  # NaN exactly where the oracle has it; the rest by value
+            assert np.array_equal(np.isnan(g_lse), np.isnan(exp_lse[op])), f"op {op}: NaN LSEs differ"
+            assert np.array_equal(np.isnan(g_out), np.isnan(exp_out[op])), f"op {op}: NaN outputs differ"
+            g_out, g_lse = np.nan_to_num(g_out, nan=0.0), np.nan_to_num(g_lse, nan=0.0)
+            exp_out[op], exp_lse[op] = np.nan_to_num(exp_out[op], nan=0.0), np.nan_to_num(exp_lse[op], nan=0.0)
+        max_out = max(max_out, np.abs(g_out - exp_out[op]).max())
+        max_lse = max(max_lse, np.abs(g_lse - exp_lse[op]).max())
     return max_out, max_lse
 
 
@@ -184,6 +192,17 @@ def test_update_out_lse_reference_shapes(gpu, name, tol):
     err_out, err_lse = _merge_case(gpu, DTYPES[name], [2, 4, 4, 2, 5], 4, 64, 256, seed=0)
     assert err_out <= tol, err_out
     assert err_lse <= 1e-3, err_lse  # tolerance on fp32 LSE
+
+
+def test_update_out_lse_nan_lse_is_a_source(gpu):
+    """Only +-inf marks an empty source (reference fused_ops.py:123): a NaN LSE takes part in the
+    merge and turns the merged LSE and output row of its (token, head) into NaN, infinite sources
+    beside it or not.  (Ops with two or more sources: a single-source op is a bit copy.)"""
+    err_out, err_lse = _merge_case(gpu, torch.bfloat16, [2, 3, 8, 2, 5], 5, 128, 128, seed=11, inf_frac=0.3,
+                                   nan_frac=0.02)
+    assert err_out <= 2e-2 and err_lse <= 1e-3, (err_out, err_lse)
+    err_out, err_lse = _merge_case(gpu, torch.float32, [4, 2], 3, 64, 64, seed=12, nan_frac=0.05)
+    assert err_out <= 2e-5 and err_lse <= 1e-3, (err_out, err_lse)
 
 
 def test_update_out_lse_nonfinite_sources(gpu):

@@ -130,6 +130,23 @@ def test_merge_nonfinite_sources_are_ignored():
     assert np.isfinite(out).all() and np.isfinite(lse).all()
 
 
+def test_merge_nan_lse_is_a_source():
+    """fused_ops.py:123 tests ``lse != -inf and lse != inf``: NaN is not an empty source, so it
+    poisons the merged (token, head) -- and nothing else."""
+    outs, lses = _rand_partials(5, S=3)
+    lses[1, 2, 7] = np.nan
+    lses[0, 1, 3], lses[2, 1, 3] = np.inf, np.nan
+    out, lse = oracle.merge_out_lse(outs, lses)
+    assert np.isnan(lse[2, 7]) and np.isnan(out[7, 2]).all() and np.isnan(lse[1, 3]) and np.isnan(out[3, 1]).all()
+    poisoned = np.zeros(lse.shape, dtype=bool)
+    poisoned[2, 7] = poisoned[1, 3] = True
+    assert np.isfinite(lse[~poisoned]).all() and np.isfinite(out[~poisoned.T]).all()
+    clean = lses.copy()
+    clean[1, 2, 7] = clean[2, 1, 3] = 0.0
+    ref = oracle.merge_out_lse(outs, clean)
+    assert np.array_equal(lse[~poisoned], ref[1][~poisoned]) and np.array_equal(out[~poisoned.T], ref[0][~poisoned.T])
+
+
 def _torch_dense(q, k, v, allowed, dout=None):
     """Textbook softmax attention in torch fp64 with autograd."""
     q = torch.tensor(q, dtype=torch.float64, requires_grad=dout is not None)

@@ -91,6 +91,45 @@ def test_static_scratch_backward_equals_workspace_backward_twice_in_a_row(gpu):
         assert (want_dq != torch.tensor(7.0, dtype=torch.bfloat16).view(torch.int16).item()).any()
 
 
+def test_static_scratch_backward_recorded_into_a_graph(gpu):
+    """The use the entry point is for: recorded into a HIP graph (after the set-up call, made outside
+    the capture, has looked up the scratch address) and replayed twice with eager work and
+    synchronisations in between; every replay gives the bits of dcp_attn_bwd."""
+    from dcp_amd import _lib
+
+    lib = _lib.load()
+    assert lib.dcp_attn_bwd_static_scratch_bytes() == 32 << 20  # set-up: resolves the address on this device
+    pr = _problem(gpu, n_rows=9, block_size=128, n_heads_q=4, n_heads_kv=2, head_dim=128, kv_blocks_per_row=4, seed=3)
+    want_dq, want_dkv = _run(lib, pr, static=False)
+    dq = torch.full_like(pr["q"], 7.0)
+    dkv = torch.full((pr["n_dkv"], pr["bs"], 2, pr["hkv"], pr["d"]), 7.0, dtype=pr["q"].dtype, device=gpu)
+    k, v = pr["kv"][:, :, 0], pr["kv"][:, :, 1]
+    dk, dv = dkv[:, :, 0], dkv[:, :, 1]
+
+    def call():
+        _lib.call("dcp_attn_bwd_static", pr["dout"].data_ptr(), pr["q"].data_ptr(), k.data_ptr(), v.data_ptr(),
+                  pr["out"].data_ptr(), pr["lse"].data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                  pr["cu_q"].data_ptr(), pr["cu_kv"].data_ptr(), pr["rng"].data_ptr(), 1, pr["q_table"].data_ptr(),
+                  pr["kv_table"].data_ptr(), pr["q_table"].data_ptr(), pr["q_table"].data_ptr(),
+                  pr["dkv_table"].data_ptr(), 0, pr["n_rows"], pr["max_kv"], pr["total_q"], pr["bs"], pr["hq"],
+                  pr["hkv"], pr["d"], pr["kv"].stride(0), pr["kv"].stride(1), dkv.stride(0), dkv.stride(1),
+                  pr["n_rows"], float(pr["d"]) ** -0.5, 0, torch.cuda.current_stream().cuda_stream)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    torch.cuda.synchronize()
+    for replay in range(2):
+        dq.fill_(7.0)
+        dkv.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dq.view(torch.int16).cpu().numpy(), want_dq), f"replay {replay}: dQ"
+        assert np.array_equal(dkv.view(torch.int16).cpu().numpy(), want_dkv), f"replay {replay}: dK/dV"
+        _run(lib, pr, static=False)  # the program's own eager work between the replays
+
+
 def test_static_scratch_backward_rejects_sizes_beyond_its_scratch(gpu):
     from dcp_amd import _lib
 
