@@ -36,6 +36,7 @@ SIGNATURES = {
     "dcp_attn_bwd_workspace_bytes": [_I, _I, _I, _I, _I],
     "dcp_attn_bwd_static": [_P] * 9 + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
     "dcp_attn_bwd_static_scratch_bytes": [],
+    "dcp_attn_bwd_select": [_I],
     "dcp_greedy_stage_selection": [_I, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P],
 }
 

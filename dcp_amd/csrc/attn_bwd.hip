@@ -51,65 +51,9 @@
 #include <algorithm>
 #include <mutex>
 
-#include "attn_common.h"
+#include "attn_bwd_params.h"
 
 namespace dcp {
-
-struct AttnBwdParams {
-  const void* dout;
-  const void* q;
-  const void* k;
-  const void* v;
-  const void* out;
-  const float* lse;
-  void* dq;
-  void* dk;
-  void* dv;
-  float* delta;      // [total_q, H]: MINUS rowsum(dO * O)
-  float* lse2;       // [total_q, H]: lse * log2(e); both written by the dQ kernel, read by the dK/dV kernel
-  int32_t* hull;     // [batch * q_tiles_per_row, 8]
-  int* tickets;      // work-item counters of the persistent dQ kernel (kTicketInts); zeroed by the hull kernel
-  const int32_t* cu_seqlens_q;
-  const int32_t* cu_seqlens_kv;
-  const int32_t* attn_range;
-  const int32_t* q_block_table;
-  const int32_t* kv_block_table;
-  const int32_t* out_block_table;
-  const int32_t* dq_block_table;
-  const int32_t* dkv_block_table;
-  const int32_t* row_order;
-  int n_ranges;
-  int batch;
-  int max_kv_blocks;
-  int total_q;
-  int block_size;
-  int n_heads_q;
-  int n_heads_kv;
-  int64_t kv_slot_stride;
-  int64_t kv_token_stride;
-  int64_t dkv_slot_stride;
-  int64_t dkv_token_stride;
-  int n_out_slots;
-  int dkv_xcd_group;     // dK/dV work items sharing one Q/dO stream (the key tiles of a row)
-  int dq_xcd_group;      // dQ work items sharing one K/V stream
-  int64_t n_dkv_items;   // batch * n_heads_kv * kv_tiles_per_row
-  int64_t n_dq_items;    // batch * n_heads_q * dq_tiles_per_row
-  int q_tiles_per_row;   // ceil(block_size / 64): query tiles of the dK/dV kernel
-  int dq_tiles_per_row;  // ceil(block_size / 128): query tiles of the dQ kernel
-  int kv_tiles_per_row;  // ceil(max_kv_blocks * block_size / 128): key tiles of the dK/dV kernel
-  float scale;
-  float scale_log2;
-};
-
-// Wave priorities by phase in the dK/dV kernel: a wave in one of its two matrix phases outranks a
-// wave doing vector work or step control on the same SIMD (-1.1 to -1.5 % on the kernel; measured
-// with the matrix phases at 1, 2 or 3 and unequal: all within 0.5 % of each other, all faster than
-// none; the same in the dQ kernel made it 1.2 % slower).
-constexpr int kPrioMatrix = 2, kPrioVector = 0;
-constexpr int kBwdBM = 64;
-constexpr int kBwdBN = 64;
-constexpr int kBwdThreads = 256;
-constexpr int kTicketInts = 16;  // one counter per XCD (the rest unused)
 
 // One wave per (row, 64-query tile).  hull[0..3] = lo0, hi0, lo1, hi1 over
 // rows with a non-empty range; hull[4..7] = the intersection (core) of the
@@ -832,13 +776,18 @@ using namespace dcp;
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// What the two-kernel backward needs: -delta and lse2 per (query, head), the hulls, the tickets.
+static size_t bwd_base_workspace_bytes(int batch, int total_q, int block_size, int n_heads_q) {
+  const size_t q_tiles = (size_t)batch * ((block_size + kBwdBM - 1) / kBwdBM);
+  return 2 * align256((size_t)total_q * n_heads_q * sizeof(float)) + align256(q_tiles * 8 * sizeof(int32_t)) +
+         align256(kTicketInts * sizeof(int32_t));
+}
+
 extern "C" size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size, int n_heads_q,
                                                int head_dim) {
   if (batch < 0 || total_q < 0 || block_size <= 0 || n_heads_q <= 0 || head_dim <= 0) return 0;
-  const size_t q_tiles = (size_t)batch * ((block_size + kBwdBM - 1) / kBwdBM);
-  (void)head_dim;
-  return 2 * align256((size_t)total_q * n_heads_q * sizeof(float)) + align256(q_tiles * 8 * sizeof(int32_t)) +
-         align256(kTicketInts * sizeof(int32_t));
+  return bwd_base_workspace_bytes(batch, total_q, block_size, n_heads_q) +
+         (bwd_fused_available() ? bwd_fused_extra_workspace_bytes(batch, block_size, n_heads_q, head_dim) : 0);
 }
 
 // Both entry points: argument checks, workspace carving, the four launches.
@@ -853,7 +802,7 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
                            int n_heads_kv, int head_dim, int64_t kv_slot_stride,
                            int64_t kv_token_stride, int64_t dkv_slot_stride,
                            int64_t dkv_token_stride, int n_out_slots, float softmax_scale,
-                           int dtype, void* stream) {
+                           int dtype, void* stream, bool allow_fused) {
   if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
     return fail(DCP_ERR_UNSUPPORTED, "attn_bwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
   if (head_dim != 64 && head_dim != 128)
@@ -882,9 +831,13 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
                 reinterpret_cast<uintptr_t>(workspace)) & 15) == 0 &&
                   ((reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) & 7) == 0,
               "attn_bwd: tensors must be 16-byte aligned (dk/dv: 8)");
-  const size_t need = dcp_attn_bwd_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim);
-  DCP_REQUIRE(workspace_bytes >= need, "attn_bwd: workspace of %zu bytes is smaller than the %zu needed",
-              workspace_bytes, need);
+  // The one-pass backward (head size 128) where the device allows it and the workspace holds its
+  // partial sums; otherwise the two-kernel one, which needs the base workspace only.
+  const size_t base = bwd_base_workspace_bytes(batch, total_q, block_size, n_heads_q);
+  const size_t extra = bwd_fused_extra_workspace_bytes(batch, block_size, n_heads_q, head_dim);
+  const bool fused = allow_fused && head_dim == 128 && bwd_fused_available() && workspace_bytes >= base + extra;
+  DCP_REQUIRE(workspace_bytes >= base, "attn_bwd: workspace of %zu bytes is smaller than the %zu needed",
+              workspace_bytes, base);
   AttnBwdParams p;
   p.dout = dout;
   p.q = q;
@@ -903,6 +856,19 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   p.hull = reinterpret_cast<int32_t*>(ws);
   ws += align256((size_t)batch * ((block_size + kBwdBM - 1) / kBwdBM) * 8 * sizeof(int32_t));
   p.tickets = reinterpret_cast<int*>(ws);
+  ws += align256(kTicketInts * sizeof(int32_t));
+  p.subs_per_row = (block_size + 31) / 32;
+  p.dq_part = nullptr;
+  p.chain = nullptr;
+  p.fault = nullptr;
+  if (fused) {
+    const size_t chunks = (size_t)batch * n_heads_q * p.subs_per_row;
+    p.dq_part = reinterpret_cast<float*>(ws);
+    ws += align256(chunks * 4096 * sizeof(float));
+    p.chain = reinterpret_cast<int*>(ws);
+    ws += align256(chunks * 4 * sizeof(int));
+    p.fault = reinterpret_cast<int*>(ws);
+  }
   p.cu_seqlens_q = cu_seqlens_q;
   p.cu_seqlens_kv = cu_seqlens_kv;
   p.attn_range = attn_range;
@@ -933,6 +899,7 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   p.dq_xcd_group = p.dq_tiles_per_row * (n_heads_q / n_heads_kv);
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * kLog2e;
+  if (fused) return launch_bwd_fused(p, dtype, (hipStream_t)stream);
   if (dtype == DCP_DTYPE_BF16)
     return head_dim == 128 ? launch_bwd<DCP_DTYPE_BF16, 128>(p, (hipStream_t)stream)
                            : launch_bwd<DCP_DTYPE_BF16, 64>(p, (hipStream_t)stream);
@@ -956,8 +923,10 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
-                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream);
+                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream, true);
 }
+
+extern "C" int dcp_attn_bwd_select(int one_pass) { return bwd_select_one_pass(one_pass); }
 
 // ---------------------------------------------------------------------------
 // The backward with its scratch inside the library, for callers that can neither allocate
@@ -1013,7 +982,8 @@ extern "C" int dcp_attn_bwd_static(const void* dout, const void* q, const void* 
                                    int64_t kv_slot_stride, int64_t kv_token_stride, int64_t dkv_slot_stride,
                                    int64_t dkv_token_stride, int n_out_slots, float softmax_scale, int dtype,
                                    void* stream) {
-  const size_t need = dcp_attn_bwd_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim);
+  (void)head_dim;
+  const size_t need = bwd_base_workspace_bytes(batch, total_q, block_size, n_heads_q);  // the two-kernel backward's
   DCP_REQUIRE(need <= (size_t)DCP_ATTN_BWD_STATIC_SCRATCH_BYTES,
               "attn_bwd_static: these sizes need %zu bytes of scratch, the built-in scratch holds %zu; "
               "use dcp_attn_bwd with a caller workspace",
@@ -1027,6 +997,6 @@ extern "C" int dcp_attn_bwd_static(const void* dout, const void* q, const void* 
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
-                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream);
+                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream, false);
 }
 

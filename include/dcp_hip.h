@@ -256,6 +256,26 @@ size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
                                     int n_heads_q, int head_dim);
 
 /*
+ * Which of its two implementations dcp_attn_bwd takes from now on (a setting of
+ * the process).  0, the default: two kernels -- a query-outer one for dQ and a
+ * key-outer one for dK/dV, seven matrix products for the backward's five, no
+ * communication between workgroups.  1: one key-outer pass (head size 128 only)
+ * in which the key tiles of a row add their shares of dQ one after the other
+ * through an fp32 partial sum in the workspace, five matrix products; it is
+ * bit-reproducible like the first, measured SLOWER on MI355X (18 ms against
+ * 12.5 ms on 65536 causal tokens), and kept as the measured alternative.  It
+ * is only taken on a device on which the workgroups of a row share an L2 (the
+ * library checks), with head size 128 and a workspace of the size
+ * dcp_attn_bwd_workspace_bytes reports WHILE 1 is selected (it then adds
+ * batch*block_size*n_heads_q*128 floats and the chain counters); otherwise
+ * the call falls back to the two kernels.  Returns the previous setting; any
+ * other argument only asks.  No counterpart in the reference, whose backward is
+ * one non-deterministic pass with atomic adds
+ * (dcp/runtime/flash_attention/executor.py:292-334).
+ */
+int dcp_attn_bwd_select(int one_pass);
+
+/*
  * dcp_attn_bwd for callers that cannot allocate device memory or carry a
  * workspace (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc).  No counterpart in the reference.  Same arguments, results
