@@ -33,6 +33,9 @@ SIGNATURES = {
     "dcp_attn_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _F, _I, _P, c_size_t, _P],
     "dcp_attn_fwd_workspace_bytes": [],
     "dcp_attn_bwd": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
+    "dcp_attn_fwd_strided": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + [_L] * 6
+                            + [_I, _F, _I, _P, c_size_t, _P],
+    "dcp_attn_bwd_strided": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 9 + [_F, _I, _P],
     "dcp_attn_bwd_workspace_bytes": [_I, _I, _I, _I, _I],
     "dcp_attn_bwd_static": [_P] * 9 + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
     "dcp_attn_bwd_static_scratch_bytes": [],

@@ -184,8 +184,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
   // loop-invariant per-lane pieces of the addresses used in the loop
   const int row_rd = Tile::row_base(c, h);
   const int col_rd = Tile::col_base(lane, true);
-  const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.block_size * q_row_stride;
-  const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.block_size * q_row_stride;
+  const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.q_slot_stride;
+  const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.out_slot_stride;
   const uint32_t tiles_at = lds_address(&tiles[0][0]);
 
   // ---- which 64-query tiles of the row see this wave's keys (the same for every head) ------
@@ -502,9 +502,9 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
   float lse2 = INFINITY, delta = 0.0f;
   {
     const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) +
-                         ((int64_t)p.q_block_table[b] * p.block_size + q_local) * q_row_stride +
+                         (int64_t)p.q_block_table[b] * p.q_slot_stride + (int64_t)q_local * q_row_stride +
                          (int64_t)head * D + h * 8;
-    const int64_t o_off = ((int64_t)o_slot * p.block_size + q_local) * q_row_stride + (int64_t)head * D + h * 8;
+    const int64_t o_off = (int64_t)o_slot * p.out_slot_stride + (int64_t)q_local * q_row_stride + (int64_t)head * D + h * 8;
     const uint16_t* dp = reinterpret_cast<const uint16_t*>(p.dout) + o_off;
     const uint16_t* op = reinterpret_cast<const uint16_t*>(p.out) + o_off;
     float dot = 0.0f;
@@ -522,7 +522,7 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
     }
     delta = -halves_sum(dot);
     if (q_valid) {
-      lse2 = p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local] * kLog2e;
+      lse2 = p.lse[(int64_t)head * p.lse_head_stride + (int64_t)o_slot * p.lse_slot_stride + q_local] * kLog2e;
       if (h == 0) {
         const int64_t qrow = (int64_t)(q_begin + q_local) * p.n_heads_q + head;
         p.delta[qrow] = delta;
@@ -716,7 +716,7 @@ __device__ __forceinline__ void attn_bwd_dq_item(KernArgs<AttnBwdParams>& p, int
 
   if (!q_valid) return;
   uint16_t* op = reinterpret_cast<uint16_t*>(p.dq) +
-                 ((int64_t)p.dq_block_table[b] * p.block_size + q_local) * q_row_stride + (int64_t)head * D + 4 * h;
+                 (int64_t)p.dq_block_table[b] * p.dq_slot_stride + (int64_t)q_local * q_row_stride + (int64_t)head * D + 4 * h;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -801,8 +801,9 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
                            int max_kv_blocks, int total_q, int block_size, int n_heads_q,
                            int n_heads_kv, int head_dim, int64_t kv_slot_stride,
                            int64_t kv_token_stride, int64_t dkv_slot_stride,
-                           int64_t dkv_token_stride, int n_out_slots, float softmax_scale,
-                           int dtype, void* stream, bool allow_fused) {
+                           int64_t dkv_token_stride, int64_t q_slot_stride, int64_t out_slot_stride,
+                           int64_t dq_slot_stride, int64_t lse_head_stride, int64_t lse_slot_stride,
+                           float softmax_scale, int dtype, void* stream, bool allow_fused) {
   if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
     return fail(DCP_ERR_UNSUPPORTED, "attn_bwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
   if (head_dim != 64 && head_dim != 128)
@@ -817,10 +818,12 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
     return fail(DCP_ERR_UNSUPPORTED, "attn_bwd: block_size %d unsupported (at most %d)", block_size, 64 * kBwdBM);
   DCP_REQUIRE(n_heads_q > 0 && n_heads_kv > 0 && n_heads_q % n_heads_kv == 0,
               "attn_bwd: n_heads_q %d must be a multiple of n_heads_kv %d", n_heads_q, n_heads_kv);
-  DCP_REQUIRE(max_kv_blocks > 0 && n_out_slots > 0, "attn_bwd: empty block tables");
+  DCP_REQUIRE(max_kv_blocks > 0, "attn_bwd: empty block tables");
   DCP_REQUIRE(kv_token_stride % 8 == 0 && kv_slot_stride % 8 == 0 && dkv_token_stride % 4 == 0 &&
-                  dkv_slot_stride % 4 == 0,
-              "attn_bwd: kv strides must be multiples of 8 elements (dkv: 4)");
+                  dkv_slot_stride % 4 == 0 && q_slot_stride % 8 == 0 && out_slot_stride % 8 == 0 && dq_slot_stride % 8 == 0,
+              "attn_bwd: q, out, dout, dq, k, v strides must be multiples of 8 elements (dk/dv: 4)");
+  DCP_REQUIRE(q_slot_stride > 0 && out_slot_stride > 0 && dq_slot_stride > 0 && lse_head_stride > 0 && lse_slot_stride > 0,
+              "attn_bwd: table strides must be positive");
   DCP_REQUIRE(dout && q && k && v && out && lse && dq && dk && dv && workspace && cu_seqlens_q &&
                   cu_seqlens_kv && attn_range && q_block_table && kv_block_table && out_block_table &&
                   dq_block_table && dkv_block_table,
@@ -889,7 +892,12 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   p.kv_token_stride = kv_token_stride;
   p.dkv_slot_stride = dkv_slot_stride;
   p.dkv_token_stride = dkv_token_stride;
-  p.n_out_slots = n_out_slots;
+  p.n_out_slots = 0;
+  p.q_slot_stride = q_slot_stride;
+  p.out_slot_stride = out_slot_stride;
+  p.dq_slot_stride = dq_slot_stride;
+  p.lse_head_stride = lse_head_stride;
+  p.lse_slot_stride = lse_slot_stride;
   p.q_tiles_per_row = (block_size + kBwdBM - 1) / kBwdBM;
   p.dq_tiles_per_row = (block_size + kDqBM - 1) / kDqBM;
   p.kv_tiles_per_row = (int)(((int64_t)max_kv_blocks * block_size + kDkvBN - 1) / kDkvBN);
@@ -919,11 +927,35 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
                             int64_t kv_token_stride, int64_t dkv_slot_stride,
                             int64_t dkv_token_stride, int n_out_slots, float softmax_scale,
                             int dtype, void* stream) {
+  DCP_REQUIRE(batch == 0 || n_out_slots > 0, "attn_bwd: empty block tables");
+  const int64_t slot = (int64_t)block_size * n_heads_q * head_dim;
   return attn_bwd_launch(dout, q, k, v, out, lse, dq, dk, dv, workspace, workspace_bytes, cu_seqlens_q,
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
-                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream, true);
+                         dkv_token_stride, slot, slot, slot, (int64_t)n_out_slots * block_size, block_size,
+                         softmax_scale, dtype, stream, true);
+}
+
+extern "C" int dcp_attn_bwd_strided(const void* dout, const void* q, const void* k, const void* v,
+                                    const void* out, const float* lse, void* dq, void* dk, void* dv,
+                                    void* workspace, size_t workspace_bytes, const int32_t* cu_seqlens_q,
+                                    const int32_t* cu_seqlens_kv, const int32_t* attn_range, int n_ranges,
+                                    const int32_t* q_block_table, const int32_t* kv_block_table,
+                                    const int32_t* out_block_table, const int32_t* dq_block_table,
+                                    const int32_t* dkv_block_table, const int32_t* row_order, int batch,
+                                    int max_kv_blocks, int total_q, int block_size, int n_heads_q,
+                                    int n_heads_kv, int head_dim, int64_t kv_slot_stride,
+                                    int64_t kv_token_stride, int64_t dkv_slot_stride,
+                                    int64_t dkv_token_stride, int64_t q_slot_stride, int64_t out_slot_stride,
+                                    int64_t dq_slot_stride, int64_t lse_head_stride, int64_t lse_slot_stride,
+                                    float softmax_scale, int dtype, void* stream) {
+  return attn_bwd_launch(dout, q, k, v, out, lse, dq, dk, dv, workspace, workspace_bytes, cu_seqlens_q,
+                         cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
+                         dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
+                         n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
+                         dkv_token_stride, q_slot_stride, out_slot_stride, dq_slot_stride, lse_head_stride,
+                         lse_slot_stride, softmax_scale, dtype, stream, true);
 }
 
 extern "C" int dcp_attn_bwd_select(int one_pass) { return bwd_select_one_pass(one_pass); }
@@ -993,10 +1025,13 @@ extern "C" int dcp_attn_bwd_static(const void* dout, const void* q, const void* 
   // Nothing in the scratch has to start at zero: delta, lse2 and the hulls are written for every
   // valid (token, head) / query tile before the kernels that read them run (and only those are
   // read), and the hull kernel zeroes the work counters on the stream.
+  DCP_REQUIRE(batch == 0 || n_out_slots > 0, "attn_bwd_static: empty block tables");
+  const int64_t slot = (int64_t)block_size * n_heads_q * head_dim;
   return attn_bwd_launch(dout, q, k, v, out, lse, dq, dk, dv, ptr, DCP_ATTN_BWD_STATIC_SCRATCH_BYTES, cu_seqlens_q,
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
-                         dkv_token_stride, n_out_slots, softmax_scale, dtype, stream, false);
+                         dkv_token_stride, slot, slot, slot, (int64_t)n_out_slots * block_size, block_size,
+                         softmax_scale, dtype, stream, false);
 }
 

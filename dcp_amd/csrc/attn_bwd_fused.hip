@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_prepare_kernel(const AttnBwdP
     const bool live = pair < n_q * H;
     const int ql = live ? pair / H : 0, head = live ? pair - ql * H : 0;
     const int q_local = qt * kBwdBM + ql;
-    const int64_t off = ((int64_t)o_slot * p.block_size + q_local) * row_stride + (int64_t)head * D + sub_lane * 8;
+    const int64_t off = (int64_t)o_slot * p.out_slot_stride + (int64_t)q_local * row_stride + (int64_t)head * D + sub_lane * 8;
     const u32x4 o = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.out) + off);
     const u32x4 g = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.dout) + off);
     float dot = 0.0f;
@@ -145,12 +145,12 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_prepare_kernel(const AttnBwdP
     if (live && sub_lane == 0) {
       const int64_t qrow = (int64_t)(q_begin + q_local) * H + head;
       p.delta[qrow] = -dot;
-      p.lse2[qrow] = p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local] * kLog2e;
+      p.lse2[qrow] = p.lse[(int64_t)head * p.lse_head_stride + (int64_t)o_slot * p.lse_slot_stride + q_local] * kLog2e;
     }
     if (nobody_visits && live) {  // no key tile sees these queries: their dQ is zero, and nobody else writes it
       const u32x4 zero = {0, 0, 0, 0};
       *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dq) +
-                                ((int64_t)p.dq_block_table[b] * p.block_size + q_local) * row_stride + (int64_t)head * D +
+                                (int64_t)p.dq_block_table[b] * p.dq_slot_stride + (int64_t)q_local * row_stride + (int64_t)head * D +
                                 sub_lane * 8) = zero;
     }
   }
@@ -277,8 +277,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_fused_kernel(const At
   const int row_rd = Tile::row_base(c, h);
   const int col_rd = Tile::col_base(lane, true);    // Q^T / dO^T in accumulator row order
   const int col_rd_k = Tile::col_base(lane, false);  // K^T slices, contraction index = key in plain order
-  const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.block_size * q_row_stride;
-  const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.block_size * q_row_stride;
+  const uint16_t* q_base = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)q_slot * p.q_slot_stride;
+  const uint16_t* do_base = reinterpret_cast<const uint16_t*>(p.dout) + (int64_t)o_slot * p.out_slot_stride;
   const uint32_t qdo_at = lds_address(&qdo[0][0]);
   // A step's tile is one 64-row tile: Q of its 32 queries in rows 0..31, dO in rows 32..63, so a
   // group load takes its lanes 0..31 from Q and 32..63 from dO.  Per lane: which array, which of
@@ -529,7 +529,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_fused_kernel(const At
       if (last) {  // the chunk is complete: scale, round, write dQ
         if (sub * BM + c < seqlen_q) {
           uint16_t* op = reinterpret_cast<uint16_t*>(p.dq) +
-                         ((int64_t)p.dq_block_table[b] * p.block_size + sub * BM + c) * q_row_stride + (int64_t)head * D +
+                         (int64_t)p.dq_block_table[b] * p.dq_slot_stride + (int64_t)(sub * BM + c) * q_row_stride + (int64_t)head * D +
                          32 * w + 4 * h;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {

@@ -45,6 +45,13 @@ struct AttnBwdParams {
   int64_t dkv_slot_stride;
   int64_t dkv_token_stride;
   int n_out_slots;
+  // element strides of a table entry: a slot of block_size tokens, or a single token when the
+  // tables address the caller's unpadded tensors directly (entries are then token offsets)
+  int64_t q_slot_stride;
+  int64_t out_slot_stride;   // out and dout
+  int64_t dq_slot_stride;
+  int64_t lse_head_stride;
+  int64_t lse_slot_stride;
   int dkv_xcd_group;     // dK/dV work items sharing one Q/dO stream (the key tiles of a row)
   int dq_xcd_group;      // dQ work items sharing one K/V stream
   int64_t n_dkv_items;   // batch * n_heads_kv * kv_tiles_per_row

@@ -62,6 +62,13 @@ struct AttnFwdParams {
   int64_t kv_slot_stride;
   int64_t kv_token_stride;
   int n_out_slots;
+  // element strides of a table entry: a slot of block_size tokens, or a single token when the
+  // tables address the caller's unpadded tensors directly (entries are then token offsets)
+  int64_t q_slot_stride;
+  int64_t out_slot_stride;
+  int64_t lse_head_stride;
+  int64_t lse_slot_stride;
+  float empty_lse;   // what the LSE of a query without a visible key reads: +inf, or the merged form -1
   int q_tiles_per_row;
   int xcd_group;     // work items per shared K/V stream
   int64_t n_items;   // batch * n_heads_q * q_tiles_per_row
@@ -146,7 +153,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) +
-                         ((int64_t)p.q_block_table[b] * p.block_size + q_local[qb]) * q_row_stride +
+                         (int64_t)p.q_block_table[b] * p.q_slot_stride + (int64_t)q_local[qb] * q_row_stride +
                          (int64_t)head * D + h * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -550,7 +557,7 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
     if (!q_valid[qb]) continue;
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     uint16_t* op = reinterpret_cast<uint16_t*>(p.out) +
-                   ((int64_t)o_slot * p.block_size + q_local[qb]) * q_row_stride + (int64_t)head * D + 4 * h;
+                   (int64_t)o_slot * p.out_slot_stride + (int64_t)q_local[qb] * q_row_stride + (int64_t)head * D + 4 * h;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -560,8 +567,8 @@ __device__ __forceinline__ void attn_fwd_item(const AttnFwdParams& p, int item) 
         *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * g) = pk;
       }
     if (h == 0) {
-      const float lse = l_tot > 0.0f ? (m_run[qb] + log2f(l_tot)) * kLn2 : INFINITY;
-      p.lse[((int64_t)head * p.n_out_slots + o_slot) * p.block_size + q_local[qb]] = lse;
+      const float lse = l_tot > 0.0f ? (m_run[qb] + log2f(l_tot)) * kLn2 : p.empty_lse;
+      p.lse[(int64_t)head * p.lse_head_stride + (int64_t)o_slot * p.lse_slot_stride + q_local[qb]] = lse;
     }
   }
 }
@@ -613,6 +620,25 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
                             int64_t kv_slot_stride, int64_t kv_token_stride, int n_out_slots,
                             float softmax_scale, int dtype, void* workspace, size_t workspace_bytes,
                             void* stream) {
+  DCP_REQUIRE(batch == 0 || n_out_slots > 0, "attn_fwd: empty block tables");
+  const int64_t slot = (int64_t)block_size * n_heads_q * head_dim;
+  return dcp_attn_fwd_strided(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_kv, attn_range, n_ranges, q_block_table,
+                              kv_block_table, out_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
+                              n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, slot, slot,
+                              (int64_t)n_out_slots * block_size, block_size, 0, softmax_scale, dtype, workspace,
+                              workspace_bytes, stream);
+}
+
+extern "C" int dcp_attn_fwd_strided(const void* q, const void* k, const void* v, void* out, float* lse,
+                                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_kv,
+                                    const int32_t* attn_range, int n_ranges, const int32_t* q_block_table,
+                                    const int32_t* kv_block_table, const int32_t* out_block_table,
+                                    const int32_t* row_order, int batch, int max_kv_blocks, int total_q,
+                                    int block_size, int n_heads_q, int n_heads_kv, int head_dim,
+                                    int64_t kv_slot_stride, int64_t kv_token_stride, int64_t q_slot_stride,
+                                    int64_t out_slot_stride, int64_t lse_head_stride, int64_t lse_slot_stride,
+                                    int merged_form, float softmax_scale, int dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
   if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
     return fail(DCP_ERR_UNSUPPORTED, "attn_fwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
   if (head_dim != 64 && head_dim != 128)
@@ -625,9 +651,11 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
               "attn_fwd: block_size %d must be a positive multiple of %d", block_size, kFwdBN);
   DCP_REQUIRE(n_heads_q > 0 && n_heads_kv > 0 && n_heads_q % n_heads_kv == 0,
               "attn_fwd: n_heads_q %d must be a multiple of n_heads_kv %d", n_heads_q, n_heads_kv);
-  DCP_REQUIRE(max_kv_blocks > 0 && n_out_slots > 0, "attn_fwd: empty block tables");
-  DCP_REQUIRE(kv_token_stride % 8 == 0 && kv_slot_stride % 8 == 0,
-              "attn_fwd: kv strides must be multiples of 8 elements");
+  DCP_REQUIRE(max_kv_blocks > 0, "attn_fwd: empty block tables");
+  DCP_REQUIRE(kv_token_stride % 8 == 0 && kv_slot_stride % 8 == 0 && q_slot_stride % 8 == 0 && out_slot_stride % 4 == 0,
+              "attn_fwd: q, k, v strides must be multiples of 8 elements (out: 4)");
+  DCP_REQUIRE(q_slot_stride > 0 && out_slot_stride > 0 && lse_head_stride > 0 && lse_slot_stride > 0,
+              "attn_fwd: table strides must be positive");
   DCP_REQUIRE(q && k && v && out && lse && cu_seqlens_q && cu_seqlens_kv && attn_range &&
                   q_block_table && kv_block_table && out_block_table,
               "attn_fwd: null argument");
@@ -660,7 +688,12 @@ extern "C" int dcp_attn_fwd(const void* q, const void* k, const void* v, void* o
   p.n_heads_kv = n_heads_kv;
   p.kv_slot_stride = kv_slot_stride;
   p.kv_token_stride = kv_token_stride;
-  p.n_out_slots = n_out_slots;
+  p.n_out_slots = 0;
+  p.q_slot_stride = q_slot_stride;
+  p.out_slot_stride = out_slot_stride;
+  p.lse_head_stride = lse_head_stride;
+  p.lse_slot_stride = lse_slot_stride;
+  p.empty_lse = merged_form ? -1.0f : INFINITY;
   // One 32-row query block per wave.  (Two per wave do not pay with this compiler: it cannot
   // keep the O^T accumulators in the AGPR half of the register file without copies and spills.)
   const int bm = 128;

@@ -72,11 +72,47 @@ def _kv_strides(k: torch.Tensor, v: torch.Tensor, name: str):
     two halves of a [n_slots, block_size, 2, n_heads_kv, D] buffer)."""
     if k.shape != v.shape or k.stride() != v.stride():
         raise ValueError(f"{name}: k and v must have the same shape and strides")
+    if k.dim() == 3:  # unpadded [tokens, n_heads_kv, D]: a table entry is a token offset
+        if k.stride(2) != 1 or k.stride(1) != k.shape[2]:
+            raise ValueError(f"{name}: k/v head and feature axes must be dense")
+        return k.stride(0), k.stride(0)
     if k.dim() != 4:
-        raise ValueError(f"{name}: k/v must be paged [n_slots, block_size, n_heads_kv, D]")
+        raise ValueError(f"{name}: k/v must be paged [n_slots, block_size, n_heads_kv, D] or unpadded [tokens, n_heads_kv, D]")
     if k.stride(3) != 1 or k.stride(2) != k.shape[3]:
         raise ValueError(f"{name}: k/v head and feature axes must be dense")
     return k.stride(0), k.stride(1)
+
+
+def _paged_or_tokens(t: torch.Tensor, name: str, block_size):
+    """``(block_size, stride of a table entry in elements)`` of a q-like tensor: paged
+    ``[n_slots, block_size, H, D]`` (a table entry is a slot) or unpadded ``[tokens, H, D]`` (a table
+    entry is a token offset; ``block_size`` then has to be given)."""
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if t.dim() == 4:
+        if block_size is not None and block_size != t.shape[1]:
+            raise ValueError(f"{name}: block size {t.shape[1]} differs from {block_size}")
+        return t.shape[1], t.shape[1] * t.shape[2] * t.shape[3]
+    if t.dim() == 3:
+        if block_size is None:
+            raise ValueError(f"{name} is unpadded [tokens, H, D]: block_size must be given")
+        return block_size, t.shape[1] * t.shape[2]
+    raise ValueError(f"{name} must be [n_slots, block_size, H, D] or [tokens, H, D]")
+
+
+def _lse_strides(lse: torch.Tensor, out: torch.Tensor, block_size: int, name: str):
+    """``(head stride, entry stride)`` of an LSE tensor that goes with ``out``: ``[H, n_slots,
+    block_size]`` beside a paged out, ``[H, tokens]`` beside an unpadded one."""
+    if lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise ValueError(f"{name} must be contiguous float32")
+    n_heads = out.shape[-2]
+    if out.dim() == 4:
+        if tuple(lse.shape) != (n_heads, out.shape[0], block_size):
+            raise ValueError(f"{name} shape {tuple(lse.shape)} does not match out")
+        return out.shape[0] * block_size, block_size
+    if tuple(lse.shape) != (n_heads, out.shape[0]):
+        raise ValueError(f"{name} shape {tuple(lse.shape)} does not match the unpadded out")
+    return out.shape[0], 1
 
 
 def _check_tables(batch, cu_seqlens_k, row_order, single, wide):
@@ -109,8 +145,13 @@ def _kernel_head_dim(head_dim: int) -> int:
     raise ValueError(f"head size {head_dim} is above the largest supported one ({KERNEL_HEAD_DIMS[-1]})")
 
 
-def _widen(t: torch.Tensor, d: int) -> torch.Tensor:
-    """A dense copy of ``t`` with its last axis zero-padded to ``d``."""
+def _widen(t: torch.Tensor, d: int, slack_tokens: int = 0) -> torch.Tensor:
+    """A dense copy of ``t`` with its last axis zero-padded to ``d``.  An unpadded tensor
+    (``[tokens, H, D]``) also gets ``slack_tokens`` zeroed tokens of storage behind its last one,
+    which the result does not show: the kernels load whole tiles past a ragged last block."""
+    if t.dim() == 3 and slack_tokens > 0:
+        wide = torch.nn.functional.pad(t, (0, d - t.shape[-1], 0, 0, 0, slack_tokens))
+        return wide[: t.shape[0]]
     return torch.nn.functional.pad(t, (0, d - t.shape[-1]))
 
 
@@ -150,6 +191,8 @@ def _flash_attn_varlen_forward(
     lse_=None,
     row_order: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
+    block_size: Optional[int] = None,
+    merged_form: bool = False,
 ):
     """Writes the row outputs into ``out_`` / ``lse_`` in place and returns
     ``(out_, lse_, None, None)`` (the reference returns
@@ -162,6 +205,12 @@ def _flash_attn_varlen_forward(
     ``row_order`` (extension): launch order of the rows, longest first.
     ``workspace`` (extension): a buffer from ``forward_workspace()``; pass one to keep the call
     allocation-free (e.g. under graph capture), otherwise it is allocated here.
+    ``block_size`` (extension): any of q, k/v, out_ (with lse_) may instead be the UNPADDED tensor
+    (``[tokens, H, D]``; lse_ ``[H, tokens]``), its block table then holding token offsets; the
+    block size, which no paged tensor may be left to tell, is then given here.  k/v must be
+    readable for ``block_size`` tokens from every table entry on (the kernel loads whole blocks).
+    ``merged_form`` (extension): queries without a visible key get ``lse = -1`` (what the merge
+    leaves for a row with no finite source) instead of ``+inf``.
     """
     _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap,
                  alibi_slopes, return_softmax)
@@ -169,19 +218,20 @@ def _flash_attn_varlen_forward(
             or out_block_table is None or out_ is None or lse_ is None:
         raise NotImplementedError(
             "only the paged, range-masked, in-place form is implemented")
-    if q.dim() != 4 or not q.is_contiguous() or not out_.is_contiguous():
-        raise ValueError("q and out_ must be contiguous [n_slots, block_size, H, D]")
-    if lse_.dtype != torch.float32 or not lse_.is_contiguous():
-        raise ValueError("lse_ must be contiguous float32 [H, n_out_slots, block_size]")
-    _, block_size, n_heads_q, head_dim = q.shape
-    n_heads_kv = k.shape[2]
+    if k.dim() == 4:
+        block_size = k.shape[1] if block_size is None else block_size
+        if block_size != k.shape[1]:
+            raise ValueError(f"k/v: block size {k.shape[1]} differs from {block_size}")
+    block_size, q_entry = _paged_or_tokens(q, "q", block_size)
+    _, out_entry = _paged_or_tokens(out_, "out_", block_size)
+    n_heads_q, head_dim = q.shape[-2], q.shape[-1]
+    n_heads_kv = k.shape[-2]
+    lse_head_stride, lse_entry = _lse_strides(lse_, out_, block_size, "lse_")
     kv_slot_stride, kv_token_stride = _kv_strides(k, v, "forward")
     n_ranges = _range_arg(attn_range, total_q)
     batch = cu_seqlens_q.numel() - 1
     _check_tables(batch, cu_seqlens_k, row_order, dict(q_block_table=q_block_table, out_block_table=out_block_table),
                   dict(kv_block_table=kv_block_table))
-    if tuple(lse_.shape) != (n_heads_q, out_.shape[0], block_size):
-        raise ValueError(f"lse_ shape {tuple(lse_.shape)} does not match out_")
     if softmax_scale is None:
         softmax_scale = head_dim ** (-0.5)
     if head_dim not in KERNEL_HEAD_DIMS:
@@ -192,9 +242,10 @@ def _flash_attn_varlen_forward(
         d = _kernel_head_dim(head_dim)
         out_wide = _widen(out_, d)  # carries the slots this call does not write
         _flash_attn_varlen_forward(
-            _widen(q, d), _widen(k, d), _widen(v, d), cu_seqlens_q, cu_seqlens_k, total_q, max_seqlen_q, max_seqlen_k,
+            _widen(q, d, block_size), _widen(k, d, block_size), _widen(v, d, block_size), cu_seqlens_q, cu_seqlens_k, total_q, max_seqlen_q, max_seqlen_k,
             dropout_p, softmax_scale, attn_range=attn_range, q_block_table=q_block_table, kv_block_table=kv_block_table,
-            out_block_table=out_block_table, out_=out_wide, lse_=lse_, row_order=row_order, workspace=workspace)
+            out_block_table=out_block_table, out_=out_wide, lse_=lse_, row_order=row_order, workspace=workspace,
+            block_size=block_size, merged_form=merged_form)
         out_.copy_(out_wide[..., :head_dim])
         return out_, lse_, None, None
     if workspace is None:
@@ -202,7 +253,7 @@ def _flash_attn_varlen_forward(
     if workspace.dtype != torch.int32 or not workspace.is_contiguous():
         raise ValueError("workspace must be a contiguous int32 tensor from forward_workspace()")
     _lib.call(
-        "dcp_attn_fwd",
+        "dcp_attn_fwd_strided",
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out_.data_ptr(), lse_.data_ptr(),
         _i32(cu_seqlens_q, "cu_seqlens_q").data_ptr(),
         _i32(cu_seqlens_k, "cu_seqlens_k").data_ptr(),
@@ -213,8 +264,8 @@ def _flash_attn_varlen_forward(
         0 if row_order is None else _i32(row_order, "row_order").data_ptr(),
         batch, kv_block_table.shape[1], int(total_q), block_size,
         n_heads_q, n_heads_kv, head_dim,
-        kv_slot_stride, kv_token_stride, out_.shape[0],
-        float(softmax_scale), dtype_code(q.dtype),
+        kv_slot_stride, kv_token_stride, q_entry, out_entry, lse_head_stride, lse_entry,
+        1 if merged_form else 0, float(softmax_scale), dtype_code(q.dtype),
         workspace.data_ptr(), workspace.numel() * 4, _stream(),
     )
     return out_, lse_, None, None
@@ -253,6 +304,7 @@ def _flash_attn_varlen_backward(
     rng_state=None,
     workspace: Optional[torch.Tensor] = None,
     row_order: Optional[torch.Tensor] = None,
+    block_size: Optional[int] = None,
 ):
     """Writes dQ into ``dq`` (slots ``dq_block_table``) and dK/dV into
     ``dk``/``dv`` (one slot per (row, kv block), ``dkv_block_table``).
@@ -267,17 +319,29 @@ def _flash_attn_varlen_backward(
     dtype, contiguous); pass a preallocated tensor to keep the call
     allocation-free (e.g. under graph capture), otherwise it is allocated
     here.
+    ``block_size`` (extension): as in the forward, q, k/v, out with dout and softmax_lse, and dq may
+    each be the unpadded tensor, addressed by token offsets in its block table.  q and dout must
+    then be readable for 64 tokens past the last row's queries (the dK/dV kernel loads whole
+    64-query tiles).  dk/dv are always paged.
     """
     _check_plain(dropout_p, causal, window_size_left, window_size_right, softcap, alibi_slopes)
     if attn_range is None or q_block_table is None or kv_block_table is None \
             or out_block_table is None or dq_block_table is None or dkv_block_table is None:
         raise NotImplementedError(
             "only the paged, range-masked form is implemented")
-    for name, t in (("q", q), ("out", out), ("dout", dout), ("dq", dq)):
-        if t.dim() != 4 or not t.is_contiguous():
-            raise ValueError(f"{name} must be contiguous [n_slots, block_size, H, D]")
-    _, block_size, n_heads_q, head_dim = q.shape
-    n_heads_kv = k.shape[2]
+    if dk.dim() != 4:
+        raise ValueError("dk/dv must be paged [n_slots, block_size, n_heads_kv, D]")
+    block_size = dk.shape[1] if block_size is None else block_size
+    if block_size != dk.shape[1] or (k.dim() == 4 and k.shape[1] != block_size):
+        raise ValueError(f"k/v/dk/dv: block sizes differ from {block_size}")
+    _, q_entry = _paged_or_tokens(q, "q", block_size)
+    _, out_entry = _paged_or_tokens(out, "out", block_size)
+    _, dq_entry = _paged_or_tokens(dq, "dq", block_size)
+    if dout.shape != out.shape or not dout.is_contiguous():
+        raise ValueError("dout must be contiguous and shaped like out (they share out_block_table)")
+    n_heads_q, head_dim = q.shape[-2], q.shape[-1]
+    n_heads_kv = k.shape[-2]
+    lse_head_stride, lse_entry = _lse_strides(softmax_lse, out, block_size, "softmax_lse")
     kv_slot_stride, kv_token_stride = _kv_strides(k, v, "backward k/v")
     dkv_slot_stride, dkv_token_stride = _kv_strides(dk, dv, "backward dk/dv")
     n_ranges = _range_arg(attn_range, total_q)
@@ -285,25 +349,21 @@ def _flash_attn_varlen_backward(
     _check_tables(batch, cu_seqlens_k, row_order,
                   dict(q_block_table=q_block_table, out_block_table=out_block_table, dq_block_table=dq_block_table),
                   dict(kv_block_table=kv_block_table, dkv_block_table=dkv_block_table))
-    if softmax_lse.dtype != torch.float32 or not softmax_lse.is_contiguous():
-        raise ValueError("softmax_lse must be contiguous float32")
-    if tuple(softmax_lse.shape) != (n_heads_q, out.shape[0], block_size):
-        raise ValueError(f"softmax_lse shape {tuple(softmax_lse.shape)} does not match out")
-    if dout.shape[0] != out.shape[0]:
-        raise ValueError("dout and out must have the same number of slots")
     if softmax_scale is None:
         softmax_scale = head_dim ** (-0.5)
     if head_dim not in KERNEL_HEAD_DIMS:
         # as in the forward: zero-padded copies at the next kernel head size; the gradients'
         # padded columns come out zero and are dropped, slots this call leaves alone are carried
         d = _kernel_head_dim(head_dim)
-        dq_wide, dk_wide, dv_wide = _widen(dq, d), _widen(dk, d), _widen(dv, d)
+        dq_wide, dk_wide, dv_wide = _widen(dq, d, block_size), _widen(dk, d), _widen(dv, d)
         _flash_attn_varlen_backward(
-            _widen(dout, d), _widen(q, d), _widen(k, d), _widen(v, d), _widen(out, d), softmax_lse, dq_wide, dk_wide,
+            _widen(dout, d, block_size), _widen(q, d, block_size), _widen(k, d, block_size), _widen(v, d, block_size),
+            _widen(out, d, block_size), softmax_lse, dq_wide, dk_wide,
             dv_wide, cu_seqlens_q, cu_seqlens_k, total_q, total_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
             causal, window_size_left, window_size_right, softcap, alibi_slopes, deterministic, attn_range=attn_range,
             q_block_table=q_block_table, kv_block_table=kv_block_table, out_block_table=out_block_table,
-            dq_block_table=dq_block_table, dkv_block_table=dkv_block_table, workspace=workspace, row_order=row_order)
+            dq_block_table=dq_block_table, dkv_block_table=dkv_block_table, workspace=workspace, row_order=row_order,
+            block_size=block_size)
         dq.copy_(dq_wide[..., :head_dim])
         dk.copy_(dk_wide[..., :head_dim])
         dv.copy_(dv_wide[..., :head_dim])
@@ -315,7 +375,7 @@ def _flash_attn_varlen_backward(
     if not workspace.is_contiguous() or ws_bytes < need:
         raise ValueError(f"workspace must be contiguous with at least {need} bytes")
     _lib.call(
-        "dcp_attn_bwd",
+        "dcp_attn_bwd_strided",
         dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
         softmax_lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
         workspace.data_ptr(), ws_bytes,
@@ -331,6 +391,7 @@ def _flash_attn_varlen_backward(
         batch, kv_block_table.shape[1], int(total_q), block_size,
         n_heads_q, n_heads_kv, head_dim,
         kv_slot_stride, kv_token_stride, dkv_slot_stride, dkv_token_stride,
-        out.shape[0], float(softmax_scale), dtype_code(q.dtype), _stream(),
+        q_entry, out_entry, dq_entry, lse_head_stride, lse_entry,
+        float(softmax_scale), dtype_code(q.dtype), _stream(),
     )
     return dq, dk, dv, None

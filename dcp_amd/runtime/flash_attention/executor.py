@@ -15,6 +15,12 @@ Differences that follow from the kernels, not from the interface:
   dKV buffer and no copy pass (reference :954-1035, :1074-1114);
 * attention rows are launched longest-first (a ``row_order`` table built in
   ``prepare``) so that ragged rows balance across the 256 CUs;
+* where a plan's block movements are plain copies (the gather of the device's own blocks into
+  slots that only the attention kernels read; a single-source scatter of a partial output, dQ or
+  summed dK/dV back into the unpadded tensors) the kernels address the unpadded ``LOCAL_*``
+  tensors themselves and the copies are not made (``direct.py``; ``direct_local`` of the
+  executor, on by default, ``DCP_DIRECT_LOCAL=0`` in the environment turns it off).  The bytes
+  in the ``LOCAL_*`` results are the same either way;
 * communication instructions run over a ``LocalFabric`` (``fabric.py``): the
   executors of several devices share one GPU and one process, the sender's
   copy kernel writes into the receiver's staging buffer and signals with a
@@ -29,6 +35,7 @@ from collections import defaultdict
 from typing import Dict, List, Optional, Tuple
 
 import math
+import os
 import numpy as np
 import torch
 
@@ -50,6 +57,7 @@ from dcp_amd.core.instructions import (
     SumInstr,
 )
 from dcp_amd.core.serialization import int_to_torch_dtype
+from dcp_amd.runtime.flash_attention.direct import DirectPlan, analyse as _analyse_direct
 from dcp_amd.flash_attn_interface import (
     _flash_attn_varlen_backward,
     _flash_attn_varlen_forward,
@@ -97,6 +105,7 @@ class AttentionExecutor(DCPExecutor):
         tp_rank: Optional[int] = None,
         use_cudagraph: bool = False,
         fabric=None,
+        direct_local: Optional[bool] = None,
     ):
         super().__init__(
             node_id=node_id,
@@ -125,10 +134,26 @@ class AttentionExecutor(DCPExecutor):
         self.mode = "Forward"
         self.use_cudagraph = use_cudagraph
         self.cuda_graph = None
+        # let the kernels address the unpadded LOCAL_* tensors where the plan only copies (direct.py)
+        self.direct_local = (os.environ.get("DCP_DIRECT_LOCAL", "1") != "0") if direct_local is None else bool(direct_local)
+        self._direct = DirectPlan()
 
     # -- buffers ---------------------------------------------------------------
     def _create_buffer(self, buffer_shape: Tuple[int, ...], buffer_dtype: int):
         return torch.zeros(*buffer_shape, dtype=int_to_torch_dtype(buffer_dtype), device="cuda")
+
+    def init_buffers(self, execution_plan: ExecutionPlan):
+        """As the base class, but the unpadded token-major tensors get one block of zeroed tokens
+        behind their last one: kernels that address them directly load whole tiles, i.e. up to a
+        block past a ragged last block (masked, but it has to be readable and finite)."""
+        for buffer_type, info in execution_plan.buffer_info.items():
+            if (self.buffers.get(buffer_type) is None and buffer_type.startswith("Local")
+                    and buffer_type not in _LSE_BUFFER_TYPES and len(info.buffer_shape) >= 2):
+                shape = tuple(info.buffer_shape)
+                per_token = int(np.prod(shape[1:]))
+                flat = torch.zeros((shape[0] + info.block_size) * per_token, dtype=int_to_torch_dtype(info.dtype), device="cuda")
+                self.buffers[buffer_type] = flat[: shape[0] * per_token].view(shape)
+        super().init_buffers(execution_plan)
 
     def log_memory_usage(self):
         total = 0.0
@@ -167,6 +192,7 @@ class AttentionExecutor(DCPExecutor):
             self.fabric.forget(self.rank)
         self.execution_plan = self.fw_exec_plan if forward else self.bw_exec_plan
         self.init_buffers(self.execution_plan)
+        self._direct = _analyse_direct(self.execution_plan) if self.direct_local and self.fabric is None else DirectPlan()
         for instr_index, instr in enumerate(self.execution_plan.instructions):
             self.instr_index = instr_index
             prep = self._prep_handlers.get(type(instr))
@@ -324,7 +350,10 @@ def _prepare_memcpy(exec: AttentionExecutor, instr: MemcpyInstr):
     head_block_size = None
     size_class = _size_classes(exec.buffer_block_strides[src.buffer_type] for src, _ in instr.src_dst_pairs
                                if src.buffer_type not in _LSE_BUFFER_TYPES)
-    for src, dst in instr.src_dst_pairs:
+    skipped = exec._direct.skip_pairs.get(exec.instr_index, ())
+    for pos, (src, dst) in enumerate(instr.src_dst_pairs):
+        if pos in skipped:  # the kernels read the source where it lies
+            continue
         src_buf, dst_buf = exec.buffers[src.buffer_type], exec.buffers[dst.buffer_type]
         src_off = cu[src.index]
         key = ((src_buf.dtype, exec.buffer_block_strides[src.buffer_type]) if src.buffer_type in _LSE_BUFFER_TYPES
@@ -408,32 +437,62 @@ def _longest_first(seqlens_kv: List[int]) -> torch.Tensor:
     return _dev(order.tolist(), torch.int32)
 
 
+def _compact_rows(instr, attn_mask: torch.Tensor):
+    """Row lengths and ranges without the rows' padding: the plan gives every row ``seqlens_q`` =
+    the padded block size and ``[0, 0)`` ranges for the padding; a kernel that writes into an
+    unpadded tensor must not see the padding as queries at all."""
+    n_tokens = [row[0].n_tokens for row in instr.q_block_table]
+    keep = np.concatenate([np.arange(n, dtype=np.int64) + start for n, start in
+                           zip(n_tokens, np.concatenate(([0], np.cumsum(instr.seqlens_q)[:-1])))]
+                          or [np.zeros(0, dtype=np.int64)])
+    return n_tokens, attn_mask[..., torch.from_numpy(keep).to(attn_mask.device)].contiguous()
+
+
+def _token_table(cu, rows, width: int = 1) -> List[List[int]]:
+    """Block table of token offsets (local block ``i`` starts at token ``local_cu_seqlens[i]``): one
+    row per attention row, from its local block index or list of indices, padded with -1."""
+    table = []
+    for row in rows:
+        blocks = row if isinstance(row, list) else [row]
+        table.append([cu[i] for i in blocks] + [-1] * (width - len(blocks)))
+    return table
+
+
 def _prepare_attn(exec: AttentionExecutor, instr: AttnInstr):
+    direct = exec._direct.operands.get(exec.instr_index, {})
+    cu = exec.execution_plan.local_cu_seqlens
+    seqlens_q, mask = instr.seqlens_q, _mask_tensor(instr.attn_mask)
+    if direct:
+        seqlens_q, mask = _compact_rows(instr, mask)
+    width = max(len(row) for row in instr.kv_block_table)
     exec._args_cache[exec.instr_index] = (
-        sum(instr.seqlens_q),
-        _cu(instr.seqlens_q),
+        sum(seqlens_q),
+        _cu(seqlens_q),
         _cu(instr.seqlens_kv),
-        _dev(_pad_block_table(instr.q_block_table), torch.int32),
-        _dev(_pad_block_table(instr.kv_block_table), torch.int32),
-        _dev(_pad_block_table(instr.out_block_table), torch.int32),
-        _mask_tensor(instr.attn_mask),
+        _dev(_token_table(cu, direct["q"]) if "q" in direct else _pad_block_table(instr.q_block_table), torch.int32),
+        _dev(_token_table(cu, direct["kv"], width) if "kv" in direct else _pad_block_table(instr.kv_block_table), torch.int32),
+        _dev(_token_table(cu, direct["out"]) if "out" in direct else _pad_block_table(instr.out_block_table), torch.int32),
+        mask,
         _longest_first(instr.seqlens_kv),
+        frozenset(direct),
         forward_workspace(),
     )
 
 
 def _kv_views(kv: torch.Tensor):
-    return kv[:, :, 0], kv[:, :, 1]
+    """K and V of a paged ``[slots, block, 2, heads, D]`` or unpadded ``[tokens, 2, heads, D]`` buffer."""
+    return (kv[:, :, 0], kv[:, :, 1]) if kv.dim() == 5 else (kv[:, 0], kv[:, 1])
 
 
 def _handle_attn(exec: AttentionExecutor, instr: AttnInstr):
     torch.cuda.nvtx.range_push("AttnInstr")
-    (total_q, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, row_order, workspace) = exec._args_cache[
+    (total_q, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, row_order, direct, workspace) = exec._args_cache[
         exec.instr_index
     ]
-    k, v = _kv_views(exec.buffers[BufferType.BUFFER_KV])
+    # an operand the plan only copies is read (written) in the unpadded tensor, by token offset
+    k, v = _kv_views(exec.buffers[BufferType.LOCAL_KV if "kv" in direct else BufferType.BUFFER_KV])
     _flash_attn_varlen_forward(
-        exec.buffers[BufferType.BUFFER_Q],
+        exec.buffers[BufferType.LOCAL_Q if "q" in direct else BufferType.BUFFER_Q],
         k,
         v,
         cu_q,
@@ -448,29 +507,37 @@ def _handle_attn(exec: AttentionExecutor, instr: AttnInstr):
         q_block_table=q_table,
         kv_block_table=kv_table,
         out_block_table=out_table,
-        out_=exec.buffers[BufferType.BUFFER_OUT],
-        lse_=exec.buffers[BufferType.BUFFER_LSE],
+        out_=exec.buffers[BufferType.LOCAL_OUT if "out" in direct else BufferType.BUFFER_OUT],
+        lse_=exec.buffers[BufferType.LOCAL_LSE if "out" in direct else BufferType.BUFFER_LSE],
         row_order=row_order,
         workspace=workspace,
+        block_size=exec.buffer_block_sizes[BufferType.BUFFER_Q],
+        merged_form="out" in direct,  # the scatter this replaces leaves lse = -1 where no key is visible
     )
     torch.cuda.nvtx.range_pop()
 
 
 def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
-    total_q = sum(instr.seqlens_q)
+    direct = exec._direct.operands.get(exec.instr_index, {})
+    cu = exec.execution_plan.local_cu_seqlens
+    seqlens_q, mask = instr.seqlens_q, _mask_tensor(instr.attn_mask)
+    if direct:
+        seqlens_q, mask = _compact_rows(instr, mask)
+    total_q = sum(seqlens_q)
     hb = exec.buffer_per_token_shape[BufferType.BUFFER_dQ][-2]
     d = exec.buffer_per_token_shape[BufferType.BUFFER_dQ][-1]
     bs = exec.buffer_block_sizes[BufferType.BUFFER_dQ]
+    width = max(len(row) for row in instr.kv_block_table)
     exec._args_cache[exec.instr_index] = (
         total_q,
         sum(instr.seqlens_kv),
-        _cu(instr.seqlens_q),
+        _cu(seqlens_q),
         _cu(instr.seqlens_kv),
-        _dev(_pad_block_table(instr.q_block_table), torch.int32),
-        _dev(_pad_block_table(instr.kv_block_table), torch.int32),
-        _dev(_pad_block_table(instr.out_block_table), torch.int32),
-        _mask_tensor(instr.attn_mask),
-        _dev(_pad_block_table(instr.dq_block_table), torch.int32),
+        _dev(_token_table(cu, direct["q"]) if "q" in direct else _pad_block_table(instr.q_block_table), torch.int32),
+        _dev(_token_table(cu, direct["kv"], width) if "kv" in direct else _pad_block_table(instr.kv_block_table), torch.int32),
+        _dev(_token_table(cu, direct["out"]) if "out" in direct else _pad_block_table(instr.out_block_table), torch.int32),
+        mask,
+        _dev(_token_table(cu, direct["dq"]) if "dq" in direct else _pad_block_table(instr.dq_block_table), torch.int32),
         _dev(_pad_block_table(instr.dkv_block_table), torch.int32),
         torch.empty(
             backward_workspace_bytes(len(instr.seqlens_q), total_q, bs, hb, d),
@@ -478,23 +545,25 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
             device="cuda",
         ),
         _longest_first(instr.seqlens_kv),
+        frozenset(direct),
     )
 
 
 def _handle_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
     torch.cuda.nvtx.range_push("AttnBackwardInstr")
     (total_q, total_kv, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, dq_table, dkv_table,
-     workspace, row_order) = exec._args_cache[exec.instr_index]
-    k, v = _kv_views(exec.buffers[BufferType.BUFFER_KV])
-    dk, dv = _kv_views(exec.buffers[BufferType.BUFFER_dKV])
+     workspace, row_order, direct) = exec._args_cache[exec.instr_index]
+    buf = exec.buffers
+    k, v = _kv_views(buf[BufferType.LOCAL_KV if "kv" in direct else BufferType.BUFFER_KV])
+    dk, dv = _kv_views(buf[BufferType.BUFFER_dKV])
     _flash_attn_varlen_backward(
-        exec.buffers[BufferType.BUFFER_dOUT],
-        exec.buffers[BufferType.BUFFER_Q],
+        buf[BufferType.LOCAL_dOUT if "out" in direct else BufferType.BUFFER_dOUT],
+        buf[BufferType.LOCAL_Q if "q" in direct else BufferType.BUFFER_Q],
         k,
         v,
-        exec.buffers[BufferType.BUFFER_OUT],
-        exec.buffers[BufferType.BUFFER_LSE],
-        exec.buffers[BufferType.BUFFER_dQ],
+        buf[BufferType.LOCAL_OUT if "out" in direct else BufferType.BUFFER_OUT],
+        buf[BufferType.LOCAL_LSE if "out" in direct else BufferType.BUFFER_LSE],
+        buf[BufferType.LOCAL_dQ if "dq" in direct else BufferType.BUFFER_dQ],
         dk,
         dv,
         cu_q,
@@ -519,6 +588,7 @@ def _handle_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
         dkv_block_table=dkv_table,
         workspace=workspace,
         row_order=row_order,
+        block_size=exec.buffer_block_sizes[BufferType.BUFFER_dKV],
     )
     torch.cuda.nvtx.range_pop()
 
@@ -544,7 +614,10 @@ def _prepare_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
     cu = exec.execution_plan.local_cu_seqlens
     width = _round_to_pow_2(max(len(op.src_buffers) for op in instr.ops))
     table, dst_offsets, n_tokens, n_srcs = [], [], [], []
-    for op in instr.ops:
+    skipped = exec._direct.skip_ops.get(exec.instr_index, ())
+    for pos, op in enumerate(instr.ops):
+        if pos in skipped:  # the attention kernel wrote this block where the op would have put it
+            continue
         srcs = [out_blk.index for out_blk, _ in op.src_buffers]
         table.append(srcs + [-1] * (width - len(srcs)))
         idx = op.dst_buffer[0].index
@@ -552,6 +625,9 @@ def _prepare_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
         n_tokens.append(op.dst_buffer[0].n_tokens)
         n_srcs.append(len(srcs))
     dst_lse = exec.buffers[types[3]]
+    if not table:
+        exec._args_cache[exec.instr_index] = None
+        return
     exec._args_cache[exec.instr_index] = (
         types,
         _dev(table, torch.int32),
@@ -565,6 +641,8 @@ def _prepare_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
 
 
 def _handle_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
+    if exec._args_cache[exec.instr_index] is None:  # every op of the plan's was a scatter the kernels made themselves
+        return
     torch.cuda.nvtx.range_push("AttnReductionInstr")
     (types, table, dst_offsets, n_tokens, n_srcs, width, dst_lse_head_stride) = exec._args_cache[
         exec.instr_index
@@ -605,9 +683,16 @@ def _prepare_sum(exec: AttentionExecutor, instr: SumInstr):
     # one launch per (dtype, size class): sums over blocks of similar sizes share it (its grid is
     # sized for the largest block, every sum carries its own element count and strides)
     size_class = _size_classes(exec.buffer_block_strides[op.src_buffers[0].buffer_type] for op in instr.ops)
-    for op in instr.ops:
+    skipped = exec._direct.skip_ops.get(exec.instr_index, ())
+    redirected = exec._direct.redirect_ops.get(exec.instr_index, {})
+    for pos, op in enumerate(instr.ops):
+        if pos in skipped:  # a kernel or an earlier sum wrote this block where the op would have put it
+            continue
         src_type = op.src_buffers[0].buffer_type
-        dst_type = op.dst_buffer.buffer_type
+        # a sum whose slot the plan only scatters back afterwards goes straight to the unpadded tensor
+        dst_block = redirected.get(pos, op.dst_buffer)
+        unpadded = bool(instr.output_is_unpadded) or pos in redirected
+        dst_type = dst_block.buffer_type
         g = groups[(exec.buffers[src_type].dtype, size_class[exec.buffer_block_strides[src_type]])]
         per_token = int(np.prod(exec.buffer_per_token_shape[src_type]))
         g["src_ptrs"].append(exec.buffers[src_type].data_ptr())
@@ -615,13 +700,13 @@ def _prepare_sum(exec: AttentionExecutor, instr: SumInstr):
         g["src_strides"].append(exec.buffer_block_strides[src_type])
         g["n_ops"].append(len(op.src_buffers))
         g["dst_ptrs"].append(exec.buffers[dst_type].data_ptr())
-        if instr.output_is_unpadded:
-            g["dst_offsets"].append(cu[op.dst_buffer.index])
+        if unpadded:
+            g["dst_offsets"].append(cu[dst_block.index])
             g["dst_strides"].append(per_token)
         else:
-            g["dst_offsets"].append(op.dst_buffer.index)
+            g["dst_offsets"].append(dst_block.index)
             g["dst_strides"].append(exec.buffer_block_strides[dst_type])
-        g["n_elems"].append(op.dst_buffer.n_tokens * per_token)
+        g["n_elems"].append(dst_block.n_tokens * per_token)
     prepared = {}
     for (dtype, _), g in groups.items():
         width = _round_to_pow_2(max(g["n_ops"]))

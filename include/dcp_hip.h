@@ -208,6 +208,48 @@ int dcp_attn_fwd(const void* q, const void* k, const void* v, void* out,
                  void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * dcp_attn_fwd with the stride of a table entry spelled out per tensor, so that
+ * the tables can address the caller's UNPADDED tensors directly instead of
+ * padded slots: entry e of q_block_table places the row's first query at
+ * q + e*q_slot_stride (elements), entry e of out_block_table its first output
+ * at out + e*out_slot_stride and its first LSE at
+ * lse + head*lse_head_stride + e*lse_slot_stride; queries of a row are
+ * n_heads_q*head_dim elements apart, their LSEs 1.  With
+ *   q_slot_stride = out_slot_stride = block_size*n_heads_q*head_dim,
+ *   lse_head_stride = n_out_slots*block_size, lse_slot_stride = block_size
+ * this is dcp_attn_fwd.  With q_slot_stride = out_slot_stride =
+ * n_heads_q*head_dim, lse_head_stride = tokens of the LSE tensor,
+ * lse_slot_stride = 1 and kv_slot_stride = kv_token_stride, every table entry
+ * is a TOKEN offset into [tokens, heads, head_dim] tensors (LSE:
+ * [n_heads_q, tokens]): what the reference's plans spell out as a gather into
+ * slots before the kernel (MemcpyInstr, executor.py:793-811) and a
+ * single-source scatter after it (executor.py:1269-1329) then needs no copy.
+ * Only the row's seqlen_q queries are read and written; key/value tiles are
+ * still loaded whole, block_size keys from every table entry on, so the k/v
+ * tensors must be readable (and finite) for block_size tokens past their last
+ * block's first token.  merged_form != 0: a query without a visible key gets
+ * lse = -1 instead of +inf (out = 0 either way), which is what the reference's
+ * merge kernel leaves for a row none of whose sources is finite
+ * (fused_ops.py:118-143) -- for outputs written where that merge would have
+ * put them.  No counterpart in the reference.
+ */
+int dcp_attn_fwd_strided(const void* q, const void* k, const void* v, void* out,
+                         float* lse, const int32_t* cu_seqlens_q,
+                         const int32_t* cu_seqlens_kv,
+                         const int32_t* attn_range, int n_ranges,
+                         const int32_t* q_block_table,
+                         const int32_t* kv_block_table,
+                         const int32_t* out_block_table,
+                         const int32_t* row_order, int batch,
+                         int max_kv_blocks, int total_q, int block_size,
+                         int n_heads_q, int n_heads_kv, int head_dim,
+                         int64_t kv_slot_stride, int64_t kv_token_stride,
+                         int64_t q_slot_stride, int64_t out_slot_stride,
+                         int64_t lse_head_stride, int64_t lse_slot_stride,
+                         int merged_form, float softmax_scale, int dtype,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Range-masked, paged, variable-length attention backward.
  * Replaces dcp_flash_attn._flash_attn_varlen_backward as called by
  * _wrapped_flash_attn_varlen_backward (executor.py:256-337) from
@@ -245,6 +287,37 @@ int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                  int64_t dkv_slot_stride, int64_t dkv_token_stride,
                  int n_out_slots, float softmax_scale, int dtype,
                  void* stream);
+
+/*
+ * dcp_attn_bwd with the stride of a table entry spelled out per tensor (see
+ * dcp_attn_fwd_strided): q_slot_stride for q, out_slot_stride for out AND dout
+ * (they share out_block_table), dq_slot_stride for dq, lse_head_stride /
+ * lse_slot_stride for lse.  With token strides the tables address the caller's
+ * unpadded q, out, dout, lse, k and v directly and dQ is written straight into
+ * the unpadded dq.  The dK/dV kernel loads whole 64-query tiles of q and dout:
+ * those tensors must be readable (and finite) for 64 tokens past the last
+ * row's queries.  dk/dv stay padded slots (a row writes whole 32-key groups).
+ * No counterpart in the reference.
+ */
+int dcp_attn_bwd_strided(const void* dout, const void* q, const void* k,
+                         const void* v, const void* out, const float* lse,
+                         void* dq, void* dk, void* dv, void* workspace,
+                         size_t workspace_bytes, const int32_t* cu_seqlens_q,
+                         const int32_t* cu_seqlens_kv,
+                         const int32_t* attn_range, int n_ranges,
+                         const int32_t* q_block_table,
+                         const int32_t* kv_block_table,
+                         const int32_t* out_block_table,
+                         const int32_t* dq_block_table,
+                         const int32_t* dkv_block_table,
+                         const int32_t* row_order, int batch, int max_kv_blocks,
+                         int total_q, int block_size, int n_heads_q,
+                         int n_heads_kv, int head_dim, int64_t kv_slot_stride,
+                         int64_t kv_token_stride, int64_t dkv_slot_stride,
+                         int64_t dkv_token_stride, int64_t q_slot_stride,
+                         int64_t out_slot_stride, int64_t dq_slot_stride,
+                         int64_t lse_head_stride, int64_t lse_slot_stride,
+                         float softmax_scale, int dtype, void* stream);
 
 /*
  * Bytes of scratch dcp_attn_bwd needs for these sizes: rowsum(dO*O) and the
