@@ -29,14 +29,26 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E
 
-# HBM bytes per launch of the backward kernel pair, from rocprofv3 --pmc runs of this
-# script (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the counter
-# reads for the 2 GiB -> 2 GiB copy kernel of the same run: x2.0 and x1.0).  Counters
-# cannot be read from inside the benchmark, so the figure is per workload and is only
-# reported for the workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {
-    "llama3_8b_causal_64k": int(((1684923.0 + 2333248.8) * 2.0 + (1304954.0 + 647948.3) * 1.0) * 1024),
-}
+def profile_traffic(workload, kernels):
+    """HBM bytes per launch of the backward's kernels, from the committed rocprofv3 summary of this
+    script (profiles/attention_<workload>_hbm_traffic.txt: a `roofline_traffic` line per kernel,
+    FETCH_SIZE and WRITE_SIZE scaled by what the counters read for a copy kernel of known size).
+    Counters cannot be read from inside the benchmark; the figure is only reported while the
+    summary covers exactly the kernels this run launched, and with the commit it was taken at."""
+    path = os.path.join(ROOT, "profiles", f"attention_{workload}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    found, source = {}, None
+    for line in open(path):
+        parts = line.split()
+        if len(parts) >= 3 and parts[0] == "roofline_traffic":
+            found[parts[1]] = int(float(parts[2]))
+        elif len(parts) >= 2 and parts[0] == "measured_at_commit":
+            source = parts[1]
+    big = {k for k in kernels if k not in ("bwd_tile_hull_kernel",)}
+    if not big or not big <= set(found):
+        return None
+    return dict(bytes=sum(found[k] for k in big), source=f"profiles/{os.path.basename(path)} @ {source}")
 
 
 # ---------------------------------------------------------------------------
@@ -511,8 +523,8 @@ def cpu_baseline(wl, fw, bw, budget_s=20.0, seed=0):
     flops = oracle.attention_flops(pairs, hb, d, "fwd+bwd")
     return dict(
         value=round(flops / elapsed / 1e12, 5), unit="TFLOP/s", cores=int(threads), kind="port",
-        sample=f"{rows} seeded q-block rows of the same schedule (fwd+bwd, dense masked attention in fp32 torch on the host, "
-               f"{elapsed:.1f} s)",
+        sample=f"{rows} seeded q-block rows of the same schedule, their shapes and masks with random N(0, 1) data "
+               f"(not the GPU run's tensors): fwd+bwd, dense masked attention in fp32 torch on the host, {elapsed:.1f} s",
     )
 
 
@@ -614,39 +626,44 @@ def main():
     kt = kernel_times(ex_f, ex_b, fw, bw, max(2, min(args.steps, 5)))
     value = flops_step / sec / 1e12
 
-    # The backward is two kernels (dK/dV key-outer, dQ query-outer) that together do
-    # the algorithmic backward work 2.5 * fwd; they are priced as one unit.
-    dkv, dq, fwd = kt["attn_bwd_dkv_kernel"], kt["attn_bwd_dq_kernel"], kt["attn_fwd_kernel"]
+    # The backward is a group of kernels that together do the algorithmic backward work
+    # 2.5 * fwd and are priced as one unit: the key-outer dK/dV kernel, a dQ kernel (one that
+    # recomputes S and dP, or one that reads the dS the dK/dV kernel stored) and the small kernel
+    # before them (range hulls; with stored dS also -delta and the base-2 log-sum-exp).
+    # Executed matrix products per kernel, of the backward's five:
+    products = {"attn_bwd_dkv_kernel": 4, "attn_bwd_dq_kernel": 3, "attn_bwd_dq_ds_kernel": 1, "attn_bwd_fused_kernel": 5,
+                "bwd_tile_hull_kernel": 0, "bwd_prepare_kernel": 0}
+    bwd = {k: v for k, v in kt.items() if k in products}
+    fwd = kt["attn_fwd_kernel"]
     # A plan that splits every row's kv blocks over several partials launches each kernel that
     # many times per step; a launch then does 1/n of the step's work on average.
-    n_launch = max(1, round(dkv["ms_per_step"] / dkv["avg_ms"]))
-    bwd_ms = dkv["avg_ms"] + dq["avg_ms"]
+    n_launch = max(1, round(fwd["ms_per_step"] / fwd["avg_ms"]))
+    bwd_ms = sum(v["avg_ms"] for v in bwd.values())
     bwd_tflops = 2.5 * flops_fwd / n_launch / (bwd_ms * 1e-3) / 1e12
     fwd_tflops = flops_fwd / n_launch / (fwd["avg_ms"] * 1e-3) / 1e12
+    traffic = profile_traffic(args.workload, set(bwd))
     roofline = dict(
-        bound="mfma", kernel="attn_bwd_dkv_kernel+attn_bwd_dq_kernel", achieved=round(bwd_tflops, 2),
+        bound="mfma", kernel="+".join(sorted(bwd)), achieved=round(bwd_tflops, 2),
         peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(bwd_tflops / PEAK_BF16_TFLOPS, 4),
-        traffic=MEASURED_TRAFFIC_BYTES.get(args.workload),
+        traffic=traffic["bytes"] if traffic else None, traffic_source=traffic["source"] if traffic else None,
         flops_per_launch=2.5 * flops_fwd / n_launch, avg_launch_ms=round(bwd_ms, 4),
     )
     extra = dict(
         attn_fwd_kernel=dict(achieved_TFLOPs=round(fwd_tflops, 2), frac_of_peak=round(fwd_tflops / PEAK_BF16_TFLOPS, 4),
                              avg_launch_ms=round(fwd["avg_ms"], 4)),
-        # executed MFMA work: dK/dV kernel 4 products (S, dP, dV, dK), dQ kernel 3 (S, dP, dQ)
-        attn_bwd_dkv_kernel=dict(executed_TFLOPs=round(2.0 * flops_fwd / n_launch / (dkv["avg_ms"] * 1e-3) / 1e12, 2),
-                                 avg_launch_ms=round(dkv["avg_ms"], 4)),
-        attn_bwd_dq_kernel=dict(executed_TFLOPs=round(1.5 * flops_fwd / n_launch / (dq["avg_ms"] * 1e-3) / 1e12, 2),
-                                avg_launch_ms=round(dq["avg_ms"], 4)),
         kernel_ms_per_step={k: round(v["ms_per_step"], 4) for k, v in sorted(kt.items())},
         mfma_only_kernel=mfma_sustained(),
     )
+    for k, v in bwd.items():
+        if products[k]:
+            extra[k] = dict(executed_TFLOPs=round(products[k] * 0.5 * flops_fwd / n_launch / (v["avg_ms"] * 1e-3) / 1e12, 2),
+                            matrix_products=products[k], avg_launch_ms=round(v["avg_ms"], 4))
     # executed MFMA rate of each attention kernel against what MFMAs sustain beside that kernel's
     # own mix of other instructions (dependency-free, no loads, no barriers)
     mix = mfma_with_instruction_mix()
-    executed = dict(attn_fwd_kernel=fwd_tflops, attn_bwd_dkv_kernel=extra["attn_bwd_dkv_kernel"]["executed_TFLOPs"],
-                    attn_bwd_dq_kernel=extra["attn_bwd_dq_kernel"]["executed_TFLOPs"])
+    executed = dict(attn_fwd_kernel=fwd_tflops, **{k: extra[k]["executed_TFLOPs"] for k in bwd if k in extra})
     extra["mfma_with_kernel_instruction_mix"] = {
-        k: dict(bound_TFLOPs=v, kernel_executed_frac_of_bound=round(executed[k] / v, 3)) for k, v in mix.items()}
+        k: dict(bound_TFLOPs=v, kernel_executed_frac_of_bound=round(executed[k] / v, 3)) for k, v in mix.items() if k in executed}
     if not args.no_movement:
         del ex_f, ex_b
         torch.cuda.empty_cache()

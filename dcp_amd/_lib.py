@@ -35,7 +35,8 @@ SIGNATURES = {
     "dcp_attn_bwd": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
     "dcp_attn_fwd_strided": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + [_L] * 6
                             + [_I, _F, _I, _P, c_size_t, _P],
-    "dcp_attn_bwd_strided": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 9 + [_F, _I, _P],
+    "dcp_attn_bwd_strided": [_P] * 10 + [c_size_t] + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 10 + [_F, _I, _P],
+    "dcp_attn_bwd_workspace_bytes_kv": [_I, _I, _L, _I, _I, _I],
     "dcp_attn_bwd_workspace_bytes": [_I, _I, _I, _I, _I],
     "dcp_attn_bwd_static": [_P] * 9 + [_P] * 3 + [_I] + [_P] * 6 + [_I] * 7 + [_L] * 4 + [_I, _F, _I, _P],
     "dcp_attn_bwd_static_scratch_bytes": [],
@@ -75,7 +76,8 @@ def load():
             fn.argtypes = argtypes
             fn.restype = {"dcp_last_error": c_char_p, "dcp_attn_bwd_workspace_bytes": c_size_t,
                           "dcp_attn_fwd_workspace_bytes": c_size_t,
-                          "dcp_attn_bwd_static_scratch_bytes": c_size_t}.get(name, c_int)
+                          "dcp_attn_bwd_static_scratch_bytes": c_size_t,
+                          "dcp_attn_bwd_workspace_bytes_kv": c_size_t}.get(name, c_int)
         _lib = lib
     return _lib
 

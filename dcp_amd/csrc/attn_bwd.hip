@@ -95,7 +95,11 @@ __global__ __launch_bounds__(64) void bwd_tile_hull_kernel(const AttnBwdParams p
 // ---------------------------------------------------------------------------
 constexpr int kDkvBN = 128;  // keys per workgroup: four waves of 32 keys each
 
-template <int DTYPE, int D>
+// WRITE_DS: the kernel also leaves dS (the storage type, zero where masked) in the workspace, for
+// the dQ kernel that contracts it with K instead of recomputing S and dP (attn_bwd_ds.hip).  A
+// piece is the dS of 64 keys x 32 queries of one head, 4 KiB, laid out as the lanes of this kernel
+// hold it: [32-key half][16-query half][key][4-query group within the 16: 2 x 2][4 queries].
+template <int DTYPE, int D, bool WRITE_DS>
 __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
   constexpr int BM = kBwdBM, BN = kDkvBN;
   constexpr int KS = D / 16;  // k-steps over the head dim
@@ -249,6 +253,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     load_async_dword(at + sc_at_second, voff, base + sc_second_bytes);
   };
 
+  // dS pieces (WRITE_DS): number of this wave's 64-key half tile among all rows' (the rows' key
+  // counts are multiples of 64), and the lane's 16 bytes within a [key][query half] plane of a piece
+  const int64_t ds_tile64 = (int64_t)(p.cu_seqlens_kv[b] / 64) + 2 * kt + (w >> 1);
+  const int ds_lane = (w & 1) * 128 + 2 * c + h;
+
   // steps: (q head of the group) x (active 64-query tile)
   int hg = 0;
   unsigned long long rem = act_mask;  // tiles of head hg still to do
@@ -258,6 +267,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
 #pragma unroll
     for (int i = 0; i < NL; ++i) request_tile(i, kv_head * group, __builtin_ctzll(rem), 0);
   }
+  if constexpr (WRITE_DS) wait_loads();  // (the wait at the top of a step counts on two stores behind the tile loads)
   while (act_mask != 0 && hg < group) {
     const int qt = __builtin_ctzll(rem);
     const bool unmasked = (unm_w >> qt) & 1;
@@ -269,8 +279,16 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     }
     const bool more = hg_next < group;
 
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed
+    if constexpr (WRITE_DS) {
+      // The tiles and scalars of this step were requested before the previous step's last two
+      // stores of dS: those may stay in flight (a full wait would sit out their trip to memory
+      // at every step; measured 9.3 ms against 7.3 ms for the kernel).
+      asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+      phase_barrier();
+    } else {
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();  // this step's tiles and scalars are in LDS; the previous step is fully consumed
+    }
     // The next step's tiles are requested one load at a time between the matrix instructions of
     // the first phases below: a burst here would hold the wave at its last load until the memory
     // pipeline has taken them all.  They are issued unconditionally, so that the step has no
@@ -286,6 +304,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     const uint64_t next_q = uniform64(reinterpret_cast<uint64_t>(q_base + off_next));
     const uint64_t next_do = uniform64(reinterpret_cast<uint64_t>(do_base + off_next));
     const uint32_t next_at = __builtin_amdgcn_readfirstlane(Tile::group_lds_at(tiles_at + 2 * (st ^ 1) * (Tile::SIZE * 2), w, 0));
+    // where this step's dS goes: the pieces of (this wave's 64-key half tile, head, the step's two 32-query sub-tiles)
+    // (a wave whose 32 keys lie past the row's last key has no piece -- its 64-key half tile would be
+    // the next row's first, or lie past the end of the workspace -- and writes its zeros into two
+    // spare pieces behind the last one instead: no branch around the stores)
+    const uint64_t ds_step = WRITE_DS ? uniform64(reinterpret_cast<uint64_t>(p.ds) +
+                                                  (((has_keys ? ((uint64_t)ds_tile64 * p.n_heads_q + (kv_head * group + hg)) * p.subs_per_row + 2 * qt
+                                                              : (uint64_t)p.ds_pieces)) << 12))
+                                      : 0;
 
     // One sub-step = this wave's 32 keys against 32 of the step's 64 queries (QI = 0, 1).
     // (A real loop, not unrolled: one copy of the body keeps the register allocation of a single
@@ -394,6 +420,17 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         pb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(pv[2], pv[3]);
         dsb[g >> 1][(g & 1) * 2] = pack2<DTYPE>(dsv[0], dsv[1]);
         dsb[g >> 1][(g & 1) * 2 + 1] = pack2<DTYPE>(dsv[2], dsv[3]);
+      }
+      if constexpr (WRITE_DS) {
+        // (non-temporal: the pieces are read once, by another kernel; they must not push the row's
+        // Q and dO tiles, which its key tiles share, out of the L2)
+        // (and through a pointer that says "global memory": built from an integer it would be a
+        // generic one, whose stores also count as LDS accesses and make every wait for an LDS
+        // operand a wait for these stores)
+        typedef __attribute__((address_space(1))) u32x4 global_u32x4;
+        global_u32x4* piece = (global_u32x4*)(ds_step + ((uint64_t)QI << 12)) + ds_lane;
+        __builtin_nontemporal_store(dsb[0], piece);
+        __builtin_nontemporal_store(dsb[1], piece + 64);
       }
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(kPrioMatrix);
@@ -765,9 +802,25 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t stream) {
   }
   {
     KernelTimer timer("attn_bwd_dkv_kernel", stream);
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<DTYPE, D>), dim3((unsigned)n_dkv), dim3(kBwdThreads), 0, stream, p);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<DTYPE, D, false>), dim3((unsigned)n_dkv), dim3(kBwdThreads), 0, stream, p);
   }
   return check_launch("attn_bwd kernels");
+}
+
+// The dK/dV kernel alone, leaving dS in the workspace (p.delta and p.lse2 come from the prepare kernel).
+int launch_bwd_dkv_writing_ds(const AttnBwdParams& p, int dtype, hipStream_t stream) {
+  const int64_t n_dkv = xcd_grid_size(p.n_dkv_items, p.dkv_xcd_group);
+  DCP_REQUIRE(n_dkv < ((int64_t)1 << 31), "attn_bwd: grid too large");
+  KernelTimer timer("attn_bwd_dkv_kernel", stream);
+  const dim3 grid((unsigned)n_dkv), block(kBwdThreads);
+  if (dtype == DCP_DTYPE_BF16) {
+    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dkv_kernel<DCP_DTYPE_BF16, 128, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_bwd_dkv_kernel<DCP_DTYPE_BF16, 64, true>), grid, block, 0, stream, p);
+  } else {
+    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dkv_kernel<DCP_DTYPE_FP16, 128, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_bwd_dkv_kernel<DCP_DTYPE_FP16, 64, true>), grid, block, 0, stream, p);
+  }
+  return check_launch("attn_bwd_dkv_kernel");
 }
 
 }  // namespace dcp
@@ -803,7 +856,7 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
                            int64_t kv_token_stride, int64_t dkv_slot_stride,
                            int64_t dkv_token_stride, int64_t q_slot_stride, int64_t out_slot_stride,
                            int64_t dq_slot_stride, int64_t lse_head_stride, int64_t lse_slot_stride,
-                           float softmax_scale, int dtype, void* stream, bool allow_fused) {
+                           int64_t total_kv, float softmax_scale, int dtype, void* stream, bool allow_fused) {
   if (dtype != DCP_DTYPE_BF16 && dtype != DCP_DTYPE_FP16)
     return fail(DCP_ERR_UNSUPPORTED, "attn_bwd: dtype %d unsupported (bf16 and fp16 only)", dtype);
   if (head_dim != 64 && head_dim != 128)
@@ -839,6 +892,11 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   const size_t base = bwd_base_workspace_bytes(batch, total_q, block_size, n_heads_q);
   const size_t extra = bwd_fused_extra_workspace_bytes(batch, block_size, n_heads_q, head_dim);
   const bool fused = allow_fused && head_dim == 128 && bwd_fused_available() && workspace_bytes >= base + extra;
+  // The backward through dS in memory where it is selected, the caller said how many keys the rows
+  // have in all and the workspace holds the dS pieces.
+  const size_t ds_bytes = bwd_ds_workspace_bytes(total_kv, block_size, n_heads_q);
+  const bool through_ds = allow_fused && !fused && bwd_select(-1) == DCP_BWD_THROUGH_DS && total_kv > 0 &&
+                          workspace_bytes >= base + ds_bytes;
   DCP_REQUIRE(workspace_bytes >= base, "attn_bwd: workspace of %zu bytes is smaller than the %zu needed",
               workspace_bytes, base);
   AttnBwdParams p;
@@ -861,9 +919,12 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   p.tickets = reinterpret_cast<int*>(ws);
   ws += align256(kTicketInts * sizeof(int32_t));
   p.subs_per_row = (block_size + 31) / 32;
+  p.head_dim = head_dim;
   p.dq_part = nullptr;
   p.chain = nullptr;
   p.fault = nullptr;
+  p.ds = through_ds ? ws : nullptr;
+  p.ds_pieces = (int64_t)(ds_bytes >> 12) - 2;  // the last two pieces are spare (waves without keys write there)
   if (fused) {
     const size_t chunks = (size_t)batch * n_heads_q * p.subs_per_row;
     p.dq_part = reinterpret_cast<float*>(ws);
@@ -908,6 +969,7 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * kLog2e;
   if (fused) return launch_bwd_fused(p, dtype, (hipStream_t)stream);
+  if (through_ds) return launch_bwd_through_ds(p, dtype, (hipStream_t)stream);
   if (dtype == DCP_DTYPE_BF16)
     return head_dim == 128 ? launch_bwd<DCP_DTYPE_BF16, 128>(p, (hipStream_t)stream)
                            : launch_bwd<DCP_DTYPE_BF16, 64>(p, (hipStream_t)stream);
@@ -933,7 +995,7 @@ extern "C" int dcp_attn_bwd(const void* dout, const void* q, const void* k, cons
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
-                         dkv_token_stride, slot, slot, slot, (int64_t)n_out_slots * block_size, block_size,
+                         dkv_token_stride, slot, slot, slot, (int64_t)n_out_slots * block_size, block_size, 0,
                          softmax_scale, dtype, stream, true);
 }
 
@@ -949,16 +1011,23 @@ extern "C" int dcp_attn_bwd_strided(const void* dout, const void* q, const void*
                                     int64_t kv_token_stride, int64_t dkv_slot_stride,
                                     int64_t dkv_token_stride, int64_t q_slot_stride, int64_t out_slot_stride,
                                     int64_t dq_slot_stride, int64_t lse_head_stride, int64_t lse_slot_stride,
-                                    float softmax_scale, int dtype, void* stream) {
+                                    int64_t total_kv, float softmax_scale, int dtype, void* stream) {
   return attn_bwd_launch(dout, q, k, v, out, lse, dq, dk, dv, workspace, workspace_bytes, cu_seqlens_q,
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
                          dkv_token_stride, q_slot_stride, out_slot_stride, dq_slot_stride, lse_head_stride,
-                         lse_slot_stride, softmax_scale, dtype, stream, true);
+                         lse_slot_stride, total_kv, softmax_scale, dtype, stream, true);
 }
 
-extern "C" int dcp_attn_bwd_select(int one_pass) { return bwd_select_one_pass(one_pass); }
+extern "C" int dcp_attn_bwd_select(int mode) { return bwd_select(mode); }
+
+extern "C" size_t dcp_attn_bwd_workspace_bytes_kv(int batch, int total_q, int64_t total_kv, int block_size,
+                                                  int n_heads_q, int head_dim) {
+  const size_t base = dcp_attn_bwd_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim);
+  if (base == 0 || bwd_select(-1) != DCP_BWD_THROUGH_DS) return base;
+  return base + bwd_ds_workspace_bytes(total_kv, block_size, n_heads_q);
+}
 
 // ---------------------------------------------------------------------------
 // The backward with its scratch inside the library, for callers that can neither allocate
@@ -1031,7 +1100,7 @@ extern "C" int dcp_attn_bwd_static(const void* dout, const void* q, const void* 
                          cu_seqlens_kv, attn_range, n_ranges, q_block_table, kv_block_table, out_block_table,
                          dq_block_table, dkv_block_table, row_order, batch, max_kv_blocks, total_q, block_size,
                          n_heads_q, n_heads_kv, head_dim, kv_slot_stride, kv_token_stride, dkv_slot_stride,
-                         dkv_token_stride, slot, slot, slot, (int64_t)n_out_slots * block_size, block_size,
+                         dkv_token_stride, slot, slot, slot, (int64_t)n_out_slots * block_size, block_size, 0,
                          softmax_scale, dtype, stream, false);
 }
 

@@ -77,7 +77,8 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_prepare_kernel(const AttnBwdP
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int b = blockIdx.x / p.q_tiles_per_row;
   const int qt = blockIdx.x - b * p.q_tiles_per_row;
-  if (blockIdx.x == 0 && tid == 0) *p.fault = 0;
+  if (blockIdx.x == 0 && tid == 0 && p.fault != nullptr) *p.fault = 0;
+  if (blockIdx.x == 0 && tid < kTicketInts) p.tickets[tid] = 0;  // for a persistent dQ kernel that follows
   const int q_begin = p.cu_seqlens_q[b];
   const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
   const int seqlen_kv = p.cu_seqlens_kv[b + 1] - p.cu_seqlens_kv[b];
@@ -108,11 +109,13 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_prepare_kernel(const AttnBwdP
     }
   }
   __syncthreads();
-  const bool nobody_visits = chain_runs(hull_lds).count() == 0;
+  // (dQ of a query tile no key tile visits is only zeroed here for the one-pass kernel, which
+  // writes dQ tile by tile; a query-outer dQ kernel writes every valid query itself)
+  const bool nobody_visits = p.chain != nullptr && chain_runs(hull_lds).count() == 0;
 
   // counters of the tile's chunks: [(row, head, 32-query sub-tile)][wave]
   const int H = p.n_heads_q;
-  for (int i = tid; i < H * 2 * 4; i += kBwdThreads) {
+  for (int i = tid; p.chain != nullptr && i < H * 2 * 4; i += kBwdThreads) {
     const int head = i / 8, rest = i - head * 8;
     const int sub = qt * 2 + rest / 4;
     if (sub < p.subs_per_row) p.chain[(((int64_t)b * H + head) * p.subs_per_row + sub) * 4 + (rest & 3)] = 0;
@@ -611,22 +614,22 @@ int probe_xcd_dealing() {
 
 namespace {
 std::mutex g_select_mu;
-int g_one_pass = -1;  // -1: not set yet (the environment decides), 0: two kernels, 1: one pass where the device allows
+int g_mode = -1;  // -1: not set yet (the environment decides); DCP_BWD_* values
 }  // namespace
 
-int bwd_select_one_pass(int on) {
+int bwd_select(int mode) {
   std::lock_guard<std::mutex> hold(g_select_mu);
-  if (g_one_pass < 0) {
-    const char* e = getenv("DCP_BWD_ONE_PASS");
-    g_one_pass = e != nullptr && e[0] == '1' ? 1 : 0;
+  if (g_mode < 0) {
+    const char* e = getenv("DCP_BWD_MODE");
+    g_mode = e != nullptr && e[0] >= '0' && e[0] <= '2' ? e[0] - '0' : DCP_BWD_THROUGH_DS;
   }
-  const int before = g_one_pass;
-  if (on == 0 || on == 1) g_one_pass = on;
+  const int before = g_mode;
+  if (mode >= 0 && mode <= 2) g_mode = mode;
   return before;
 }
 
 bool bwd_fused_available() {
-  if (bwd_select_one_pass(-1) == 0) return false;
+  if (bwd_select(-1) != DCP_BWD_ONE_PASS) return false;
   static std::mutex mu;
   static int cached[64];  // 0: not asked yet, 1: yes, 2: no
   std::lock_guard<std::mutex> hold(mu);
@@ -642,16 +645,23 @@ size_t bwd_fused_extra_workspace_bytes(int batch, int block_size, int n_heads_q,
   return align256(chunks * kChunkFloats * sizeof(float)) + align256(chunks * 4 * sizeof(int)) + 256;
 }
 
+int launch_bwd_prepare(const AttnBwdParams& p, int dtype, hipStream_t stream) {
+  KernelTimer timer("bwd_prepare_kernel", stream);
+  const dim3 grid(p.batch * p.q_tiles_per_row), block(kBwdThreads);
+  if (dtype == DCP_DTYPE_BF16) {
+    if (p.head_dim == 128) hipLaunchKernelGGL((bwd_prepare_kernel<DCP_DTYPE_BF16, 128>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((bwd_prepare_kernel<DCP_DTYPE_BF16, 64>), grid, block, 0, stream, p);
+  } else {
+    if (p.head_dim == 128) hipLaunchKernelGGL((bwd_prepare_kernel<DCP_DTYPE_FP16, 128>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((bwd_prepare_kernel<DCP_DTYPE_FP16, 64>), grid, block, 0, stream, p);
+  }
+  return check_launch("bwd_prepare_kernel");
+}
+
 int launch_bwd_fused(const AttnBwdParams& p, int dtype, hipStream_t stream) {
   const int64_t n_wg = xcd_grid_size(p.n_dkv_items, p.dkv_xcd_group);
   DCP_REQUIRE(n_wg < ((int64_t)1 << 31), "attn_bwd: grid too large");
-  {
-    KernelTimer timer("bwd_prepare_kernel", stream);
-    if (dtype == DCP_DTYPE_BF16)
-      hipLaunchKernelGGL((bwd_prepare_kernel<DCP_DTYPE_BF16, 128>), dim3(p.batch * p.q_tiles_per_row), dim3(kBwdThreads), 0, stream, p);
-    else
-      hipLaunchKernelGGL((bwd_prepare_kernel<DCP_DTYPE_FP16, 128>), dim3(p.batch * p.q_tiles_per_row), dim3(kBwdThreads), 0, stream, p);
-  }
+  if (const int e = launch_bwd_prepare(p, dtype, stream)) return e;
   {
     KernelTimer timer("attn_bwd_fused_kernel", stream);
     if (dtype == DCP_DTYPE_BF16)

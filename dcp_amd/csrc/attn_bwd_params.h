@@ -24,6 +24,10 @@ struct AttnBwdParams {
   int* chain;        // [batch * n_heads_q * subs_per_row][4]: links of the chunk's chain done so far, per wave
   int* fault;        // [0]: raised by a wave whose wait for a chain link ran into the spin limit; [1]: unused word
   int subs_per_row;  // ceil(block_size / 32)
+  // the dS-through-memory backward only (attn_bwd_ds.hip):
+  void* ds;          // [total_kv / 64][n_heads_q][subs_per_row] pieces of 4 KiB: dS of 64 keys x 32 queries
+  int64_t ds_pieces;  // pieces in use; two spare ones follow
+  int head_dim;
   const int32_t* cu_seqlens_q;
   const int32_t* cu_seqlens_kv;
   const int32_t* attn_range;
@@ -73,17 +77,24 @@ constexpr int kBwdBN = 64;
 constexpr int kBwdThreads = 256;
 constexpr int kTicketInts = 16;  // one counter per XCD (the rest unused)
 
+// The backward through dS in memory: prepare (hulls, -delta, lse2), the dK/dV kernel writing dS, the
+// dQ kernel that reads it back (attn_bwd_ds.hip); the pieces it is made of live in three files.
+int launch_bwd_through_ds(const AttnBwdParams& p, int dtype, hipStream_t stream);
+int launch_bwd_prepare(const AttnBwdParams& p, int dtype, hipStream_t stream);
+int launch_bwd_dkv_writing_ds(const AttnBwdParams& p, int dtype, hipStream_t stream);
+size_t bwd_ds_workspace_bytes(int64_t total_kv, int block_size, int n_heads_q);
+
 // The one-pass backward (prepare + fused kernel) for head size 128; p.hull, p.delta, p.lse2,
 // p.dq_part, p.chain and p.fault point into the workspace.
 int launch_bwd_fused(const AttnBwdParams& p, int dtype, hipStream_t stream);
 // Bytes of workspace the one-pass backward needs beyond the two-kernel one's.
 size_t bwd_fused_extra_workspace_bytes(int batch, int block_size, int n_heads_q, int head_dim);
 // Whether dcp_attn_bwd takes the one-pass backward: it has been selected (dcp_attn_bwd_select, or
-// DCP_BWD_ONE_PASS=1 in the environment; the default is the two-kernel backward, which is the
-// faster one) and the current device deals the workgroups of a grid to its 8 XCDs in turn -- the chain relies on the
-// key tiles of a row sharing an L2 (checked once per device by a small kernel).
+// DCP_BWD_MODE in the environment) and the current device deals the workgroups of a grid to its 8
+// XCDs in turn -- the chain relies on the key tiles of a row sharing an L2 (checked once per device
+// by a small kernel).
 bool bwd_fused_available();
-// Sets the selection (0 / 1; anything else only asks) and returns what it was.
-int bwd_select_one_pass(int on);
+// Sets the selection (a DCP_BWD_* value; anything else only asks) and returns what it was.
+int bwd_select(int mode);
 
 }  // namespace dcp

@@ -245,6 +245,14 @@ struct KvTile {
                  : "s"(lds_at), "v"(off0), "s"(base)
                  : "memory");
   }
+  // The same for data that is read once (non-temporal: it takes no room in the L2 that the shared
+  // tiles need).
+  __device__ static __forceinline__ void load_group_at_streaming(uint32_t lds_at, uint64_t base, uint32_t off0) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                 :
+                 : "s"(lds_at), "v"(off0), "s"(base)
+                 : "memory");
+  }
   // LDS byte address of the wave's group load i, and the global byte step between group loads (its
   // rows lie four rows below those of load i - 1)
   __device__ static __forceinline__ uint32_t group_lds_at(uint32_t tile_at, int wave, int i) {

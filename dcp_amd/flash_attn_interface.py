@@ -28,10 +28,12 @@ __all__ = [
 ]
 
 
-def backward_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim) -> int:
-    """Scratch bytes ``_flash_attn_varlen_backward`` needs for these sizes."""
-    return int(_lib.load().dcp_attn_bwd_workspace_bytes(
-        int(batch), int(total_q), int(block_size), int(n_heads_q), int(head_dim)))
+def backward_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim, total_k=0) -> int:
+    """Scratch bytes ``_flash_attn_varlen_backward`` needs for these sizes with the backward that is
+    selected now (``dcp_attn_bwd_select``).  ``total_k``: the sum of the rows' key counts; without
+    it the backward that keeps dS in memory cannot be taken (the call then recomputes instead)."""
+    return int(_lib.load().dcp_attn_bwd_workspace_bytes_kv(
+        int(batch), int(total_q), int(total_k), int(block_size), int(n_heads_q), int(head_dim)))
 
 
 def forward_workspace(device="cuda") -> torch.Tensor:
@@ -368,9 +370,11 @@ def _flash_attn_varlen_backward(
         dk.copy_(dk_wide[..., :head_dim])
         dv.copy_(dv_wide[..., :head_dim])
         return dq, dk, dv, None
+    # (a caller's workspace may be the smaller one of the recomputing backward: the call then takes that one)
     need = backward_workspace_bytes(batch, int(total_q), block_size, n_heads_q, head_dim)
     if workspace is None:
-        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        workspace = torch.empty(backward_workspace_bytes(batch, int(total_q), block_size, n_heads_q, head_dim, int(total_k or 0)),
+                                dtype=torch.uint8, device=q.device)
     ws_bytes = workspace.numel() * workspace.element_size()
     if not workspace.is_contiguous() or ws_bytes < need:
         raise ValueError(f"workspace must be contiguous with at least {need} bytes")
@@ -391,7 +395,7 @@ def _flash_attn_varlen_backward(
         batch, kv_block_table.shape[1], int(total_q), block_size,
         n_heads_q, n_heads_kv, head_dim,
         kv_slot_stride, kv_token_stride, dkv_slot_stride, dkv_token_stride,
-        q_entry, out_entry, dq_entry, lse_head_stride, lse_entry,
+        q_entry, out_entry, dq_entry, lse_head_stride, lse_entry, int(total_k or 0),
         float(softmax_scale), dtype_code(q.dtype), _stream(),
     )
     return dq, dk, dv, None

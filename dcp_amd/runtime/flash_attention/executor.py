@@ -540,7 +540,7 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
         _dev(_token_table(cu, direct["dq"]) if "dq" in direct else _pad_block_table(instr.dq_block_table), torch.int32),
         _dev(_pad_block_table(instr.dkv_block_table), torch.int32),
         torch.empty(
-            backward_workspace_bytes(len(instr.seqlens_q), total_q, bs, hb, d),
+            backward_workspace_bytes(len(instr.seqlens_q), total_q, bs, hb, d, sum(instr.seqlens_kv)),
             dtype=torch.uint8,
             device="cuda",
         ),

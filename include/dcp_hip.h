@@ -290,7 +290,9 @@ int dcp_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
 
 /*
  * dcp_attn_bwd with the stride of a table entry spelled out per tensor (see
- * dcp_attn_fwd_strided): q_slot_stride for q, out_slot_stride for out AND dout
+ * dcp_attn_fwd_strided) and with total_kv, the sum of the rows' key counts
+ * (cu_seqlens_kv[batch], which the host side of the call cannot read; 0 = not
+ * known, which rules DCP_BWD_THROUGH_DS out): q_slot_stride for q, out_slot_stride for out AND dout
  * (they share out_block_table), dq_slot_stride for dq, lse_head_stride /
  * lse_slot_stride for lse.  With token strides the tables address the caller's
  * unpadded q, out, dout, lse, k and v directly and dQ is written straight into
@@ -317,7 +319,8 @@ int dcp_attn_bwd_strided(const void* dout, const void* q, const void* k,
                          int64_t dkv_token_stride, int64_t q_slot_stride,
                          int64_t out_slot_stride, int64_t dq_slot_stride,
                          int64_t lse_head_stride, int64_t lse_slot_stride,
-                         float softmax_scale, int dtype, void* stream);
+                         int64_t total_kv, float softmax_scale, int dtype,
+                         void* stream);
 
 /*
  * Bytes of scratch dcp_attn_bwd needs for these sizes: rowsum(dO*O) and the
@@ -329,24 +332,45 @@ size_t dcp_attn_bwd_workspace_bytes(int batch, int total_q, int block_size,
                                     int n_heads_q, int head_dim);
 
 /*
- * Which of its two implementations dcp_attn_bwd takes from now on (a setting of
- * the process).  0, the default: two kernels -- a query-outer one for dQ and a
- * key-outer one for dK/dV, seven matrix products for the backward's five, no
- * communication between workgroups.  1: one key-outer pass (head size 128 only)
- * in which the key tiles of a row add their shares of dQ one after the other
- * through an fp32 partial sum in the workspace, five matrix products; it is
- * bit-reproducible like the first, measured SLOWER on MI355X (18 ms against
- * 12.5 ms on 65536 causal tokens), and kept as the measured alternative.  It
- * is only taken on a device on which the workgroups of a row share an L2 (the
- * library checks), with head size 128 and a workspace of the size
- * dcp_attn_bwd_workspace_bytes reports WHILE 1 is selected (it then adds
- * batch*block_size*n_heads_q*128 floats and the chain counters); otherwise
- * the call falls back to the two kernels.  Returns the previous setting; any
- * other argument only asks.  No counterpart in the reference, whose backward is
- * one non-deterministic pass with atomic adds
+ * Which of its implementations the backward takes from now on (a setting of the
+ * process; DCP_BWD_MODE=0/1/2 in the environment presets it).  All three are
+ * free of atomics and bit-reproducible.
+ *  DCP_BWD_TWO_KERNELS  a query-outer kernel for dQ and a key-outer one for
+ *      dK/dV, each recomputing S and dP: seven matrix products for the
+ *      backward's five, nothing but the small workspace.
+ *  DCP_BWD_ONE_PASS  one key-outer pass (head size 128 only) in which the key
+ *      tiles of a row add their shares of dQ one after the other through an
+ *      fp32 partial sum in the workspace: five products.  Measured SLOWER on
+ *      MI355X (18 ms against 12.5 ms on 65536 causal tokens) and kept as the
+ *      measured alternative; only taken on a device on which the workgroups of
+ *      a row share an L2 (the library checks).
+ *  DCP_BWD_THROUGH_DS  (the default) the key-outer kernel also stores dS, 2 bytes
+ *      per (query, key) pair and head of every tile pair it visits, and the dQ
+ *      kernel reads it back instead of recomputing it: five products, paid for
+ *      with HBM traffic and workspace (4 KiB per 64 keys x 32 queries x head:
+ *      21 GB on 65536 causal tokens with 32 heads).  Only
+ *      dcp_attn_bwd_strided, which is told total_kv, can take it.
+ * A mode whose workspace the caller did not provide (see
+ * dcp_attn_bwd_workspace_bytes_kv) or whose conditions do not hold falls back
+ * to DCP_BWD_TWO_KERNELS.  Returns the previous setting; any other argument
+ * only asks.  No counterpart in the reference, whose backward is one
+ * non-deterministic pass with atomic adds
  * (dcp/runtime/flash_attention/executor.py:292-334).
  */
-int dcp_attn_bwd_select(int one_pass);
+#define DCP_BWD_TWO_KERNELS 0
+#define DCP_BWD_ONE_PASS 1
+#define DCP_BWD_THROUGH_DS 2
+int dcp_attn_bwd_select(int mode);
+
+/*
+ * Bytes of workspace the SELECTED backward needs for these sizes, total_kv =
+ * the sum of the rows' key counts (cu_seqlens_kv[batch]); what
+ * dcp_attn_bwd_workspace_bytes reports plus, for DCP_BWD_THROUGH_DS, the dS
+ * pieces, and for DCP_BWD_ONE_PASS the partial sums and chain counters.
+ */
+size_t dcp_attn_bwd_workspace_bytes_kv(int batch, int total_q, int64_t total_kv,
+                                       int block_size, int n_heads_q,
+                                       int head_dim);
 
 /*
  * dcp_attn_bwd for callers that cannot allocate device memory or carry a
