@@ -427,11 +427,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         // (and through a pointer that says "global memory": built from an integer it would be a
         // generic one, whose stores also count as LDS accesses and make every wait for an LDS
         // operand a wait for these stores)
-        typedef __attribute__((address_space(1))) u32x4 global_u32x4;
-        global_u32x4* piece = (global_u32x4*)(ds_step + ((uint64_t)QI << 12)) + ds_lane;
-        __builtin_nontemporal_store(dsb[0], piece);
-        __builtin_nontemporal_store(dsb[1], piece + 64);
+        // The two stores go out one at a time between the matrix instructions of the second phase
+        // (below), like the tile loads of the first.
       }
+      typedef __attribute__((address_space(1))) u32x4 global_u32x4;
+      global_u32x4* piece = (global_u32x4*)(ds_step + ((uint64_t)QI << 12)) + ds_lane;
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(kPrioMatrix);
 #pragma unroll
@@ -445,6 +445,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         if (i & 1) dk_acc[d] = mfma_32x32x16<DTYPE>(buf[o % RING], dsb[s2], dk_acc[d]);
         else dv_acc[d] = mfma_32x32x16<DTYPE>(buf[o % RING], pb[s2], dv_acc[d]);
         if (o + AHEAD < NS) buf[(o + AHEAD) % RING] = entry(o + AHEAD);
+        if constexpr (WRITE_DS) {
+          if (i == 3) __builtin_nontemporal_store(dsb[0], piece);
+          if (i == 9) __builtin_nontemporal_store(dsb[1], piece + 64);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     };
