@@ -447,7 +447,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         if (o + AHEAD < NS) buf[(o + AHEAD) % RING] = entry(o + AHEAD);
         if constexpr (WRITE_DS) {
           if (i == 3) __builtin_nontemporal_store(dsb[0], piece);
-          if (i == 9) __builtin_nontemporal_store(dsb[1], piece + 64);
+          if (i == 2 * DT + 1) __builtin_nontemporal_store(dsb[1], piece + 64);  // (2 * 2 * DT iterations)
         }
         __builtin_amdgcn_sched_barrier(0);
       }

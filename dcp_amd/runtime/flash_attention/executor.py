@@ -193,12 +193,30 @@ class AttentionExecutor(DCPExecutor):
         self.execution_plan = self.fw_exec_plan if forward else self.bw_exec_plan
         self.init_buffers(self.execution_plan)
         self._direct = _analyse_direct(self.execution_plan) if self.direct_local and self.fabric is None else DirectPlan()
+        self._bwd_workspace_bytes = 0
+        self._bwd_workspace = None
         for instr_index, instr in enumerate(self.execution_plan.instructions):
             self.instr_index = instr_index
             prep = self._prep_handlers.get(type(instr))
             if prep is not None:
                 prep(self, instr)
+        if self._bwd_workspace_bytes:
+            self._bwd_workspace = torch.empty(self._bwd_workspace_bytes, dtype=torch.uint8, device="cuda")
         torch.cuda.nvtx.range_pop()
+
+    def _reserve_backward_workspace(self, batch, total_q, block_size, n_heads, head_dim, total_kv) -> int:
+        """Bytes of the backward scratch one instruction uses.  The plan's backward instructions run one
+        after another on one stream and share a single buffer, sized for the largest.  The backward
+        that keeps dS in memory needs 2 * block_size * n_heads bytes per key of the launch; past
+        ``DCP_BWD_DS_MAX_BYTES`` (default: a quarter of the device's memory) the instruction gets the
+        small scratch instead and the library recomputes."""
+        nbytes = backward_workspace_bytes(batch, total_q, block_size, n_heads, head_dim, total_kv)
+        limit = os.environ.get("DCP_BWD_DS_MAX_BYTES")
+        limit = int(limit) if limit else torch.cuda.get_device_properties(torch.cuda.current_device()).total_memory // 4
+        if nbytes > limit:
+            nbytes = backward_workspace_bytes(batch, total_q, block_size, n_heads, head_dim, 0)
+        self._bwd_workspace_bytes = max(self._bwd_workspace_bytes, nbytes)
+        return nbytes
 
     def switch_to_backward(self):
         self.mode = "Backward"
@@ -539,11 +557,7 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
         mask,
         _dev(_token_table(cu, direct["dq"]) if "dq" in direct else _pad_block_table(instr.dq_block_table), torch.int32),
         _dev(_pad_block_table(instr.dkv_block_table), torch.int32),
-        torch.empty(
-            backward_workspace_bytes(len(instr.seqlens_q), total_q, bs, hb, d, sum(instr.seqlens_kv)),
-            dtype=torch.uint8,
-            device="cuda",
-        ),
+        exec._reserve_backward_workspace(len(instr.seqlens_q), total_q, bs, hb, d, sum(instr.seqlens_kv)),
         _longest_first(instr.seqlens_kv),
         frozenset(direct),
     )
@@ -552,7 +566,8 @@ def _prepare_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
 def _handle_attn_bw(exec: AttentionExecutor, instr: AttnBackwardInstr):
     torch.cuda.nvtx.range_push("AttnBackwardInstr")
     (total_q, total_kv, cu_q, cu_kv, q_table, kv_table, out_table, attn_mask, dq_table, dkv_table,
-     workspace, row_order, direct) = exec._args_cache[exec.instr_index]
+     workspace_bytes, row_order, direct) = exec._args_cache[exec.instr_index]
+    workspace = exec._bwd_workspace[:workspace_bytes]
     buf = exec.buffers
     k, v = _kv_views(buf[BufferType.LOCAL_KV if "kv" in direct else BufferType.BUFFER_KV])
     dk, dv = _kv_views(buf[BufferType.BUFFER_dKV])
