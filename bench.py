@@ -200,7 +200,7 @@ def load_probes():
         P, I = ctypes.c_void_p, ctypes.c_int
         lib.bench_mfma_probe.argtypes = [P, P, I, I, I, P, P]
         lib.bench_mfma_mix_probe.argtypes = [P, P, I, I, I, P, P]
-        lib.bench_hbm_stream_probe.argtypes = [P, P, I, ctypes.c_size_t, P]
+        lib.bench_hbm_stream_probe.argtypes = [P, P, I, ctypes.c_size_t, P, ctypes.c_size_t, P]
         lib.bench_probe_last_error.restype = ctypes.c_char_p
         _PROBES = lib
     return _PROBES
@@ -390,8 +390,11 @@ def movement_microbench(iters=5, bs=512):
     stream_gbps = {}
     stream = torch.cuda.current_stream().cuda_stream
     per_stream = tokens * heads * d * 2  # 2 GiB
+    # (1 read: the copy's permutation of 4 MiB blocks; 4 reads: the very table of the merge and the sum)
+    tables = {1: i32(perm), 4: table}
     for ns in (1, 4):
-        call = lambda: call_probe("bench_hbm_stream_probe", outs.data_ptr(), dst_out.data_ptr(), ns, per_stream, stream)
+        call = lambda: call_probe("bench_hbm_stream_probe", outs.data_ptr(), dst_out.data_ptr(), ns, per_stream,
+                                  tables[ns].data_ptr(), numel * 2, stream)
         call()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()

@@ -128,27 +128,36 @@ __global__ __launch_bounds__(kProbeThreads, 2) void mfma_mix_probe_kernel(const 
   out[2 + (size_t)blockIdx.x * kProbeThreads + threadIdx.x] = r;
 }
 
-// Plain streaming kernel for the HBM roofline discussion: NS equally long input streams are
-// added 16 bytes at a time (non-temporal loads) and written once (non-temporal store).  What
-// this reaches is the practical ceiling for the gather / merge / sum kernels at the same
-// read : write mix.
+// Plain streaming kernel for the HBM roofline discussion: NS input streams are added 16 bytes at a
+// time (non-temporal loads) and written once (non-temporal store), one wave per workgroup and one
+// 16-byte word per lane and stream: 1 KiB per stream and workgroup, the shape that measured fastest
+// (256 lanes x 1 word: 3 % slower with one stream, 4 % with four; two words per lane: 10 % slower).
+// Every stream is a sequence of blocks of `words_per_block` words; with a table, block b of stream
+// s is block table[b * NS + s] of `src` (the gather / merge / sum kernels read their sources through
+// such tables: where the blocks lie decides how the streams fall on the memory channels); without
+// one the streams lie end to end.  What this reaches is the practical ceiling for those kernels at
+// the same read : write mix.
 template <int NS>
-__global__ __launch_bounds__(256) void hbm_stream_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
-                                                         size_t words_per_stream) {
-  constexpr int UNR = 2;
-  const size_t base = (size_t)blockIdx.x * 256 * UNR + threadIdx.x;
-  u32x4 v[NS][UNR];
+__global__ __launch_bounds__(64) void hbm_stream_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                        size_t words_per_stream, const int32_t* __restrict__ table,
+                                                        unsigned chunks_per_block) {
+  const size_t chunk = blockIdx.x;
+  const size_t base = chunk * 64 + threadIdx.x;
+  u32x4 v[NS];
+  if (table) {
+    const size_t b = chunk / chunks_per_block;
+    const size_t within = (chunk - b * chunks_per_block) * 64 + threadIdx.x;
 #pragma unroll
-  for (int s = 0; s < NS; ++s)
+    for (int s = 0; s < NS; ++s)
+      v[s] = __builtin_nontemporal_load(src + (size_t)table[b * NS + s] * chunks_per_block * 64 + within);
+  } else {
 #pragma unroll
-    for (int u = 0; u < UNR; ++u) v[s][u] = __builtin_nontemporal_load(src + s * words_per_stream + base + u * 256);
-#pragma unroll
-  for (int u = 0; u < UNR; ++u) {
-    u32x4 acc = v[0][u];
-#pragma unroll
-    for (int s = 1; s < NS; ++s) acc += v[s][u];
-    __builtin_nontemporal_store(acc, dst + base + u * 256);
+    for (int s = 0; s < NS; ++s) v[s] = __builtin_nontemporal_load(src + s * words_per_stream + base);
   }
+  u32x4 acc = v[0];
+#pragma unroll
+  for (int s = 1; s < NS; ++s) acc += v[s];
+  __builtin_nontemporal_store(acc, dst + base);
 }
 
 }  // namespace dcp
@@ -157,26 +166,31 @@ using namespace dcp;
 
 extern "C" const char* bench_probe_last_error(void) { return dcp::last_error_buffer(); }
 
-// Adds `n_streams` (1, 2 or 4) equally long input streams, laid end to end in `src`, 16 bytes at
-// a time and writes the sum to `dst`: n_streams reads and one write of `bytes_per_stream` (a
-// multiple of 8192) each.  Time it with events on `stream`.
+// Adds `n_streams` (1, 2 or 4) equally long input streams 16 bytes at a time and writes the sum to
+// `dst`: n_streams reads and one write of `bytes_per_stream` each.  `block_table` null: the streams lie
+// end to end in `src`.  Otherwise a stream is made of blocks of `block_bytes` (a multiple of 1024 that
+// divides bytes_per_stream) and block b of stream s is block block_table[b * n_streams + s] of `src`
+// (device memory, int32).  Time it with events on `stream`.
 extern "C" int bench_hbm_stream_probe(const void* src, void* dst, int n_streams, size_t bytes_per_stream,
-                                    void* stream) {
+                                      const int32_t* block_table, size_t block_bytes, void* stream) {
   DCP_REQUIRE(src && dst, "hbm_stream_probe: null argument");
-  DCP_REQUIRE(bytes_per_stream > 0 && bytes_per_stream % (256 * 2 * 16) == 0,
-              "hbm_stream_probe: bytes_per_stream must be a positive multiple of 8192");
-  DCP_REQUIRE(bytes_per_stream / 8192 < ((size_t)1 << 31), "hbm_stream_probe: stream too long");
+  DCP_REQUIRE(bytes_per_stream > 0 && bytes_per_stream % 1024 == 0,
+              "hbm_stream_probe: bytes_per_stream must be a positive multiple of 1024");
+  DCP_REQUIRE(bytes_per_stream / 1024 < ((size_t)1 << 31), "hbm_stream_probe: stream too long");
+  DCP_REQUIRE(!block_table || (block_bytes > 0 && block_bytes % 1024 == 0 && bytes_per_stream % block_bytes == 0),
+              "hbm_stream_probe: block_bytes must be a multiple of 1024 that divides bytes_per_stream");
   const size_t words = bytes_per_stream / 16;
-  dim3 grid((unsigned)(bytes_per_stream / 8192)), block(256);
+  const unsigned chunks_per_block = block_table ? (unsigned)(block_bytes / 1024) : 1;
+  dim3 grid((unsigned)(bytes_per_stream / 1024)), block(64);
   switch (n_streams) {
     case 1:
-      hipLaunchKernelGGL(hbm_stream_kernel<1>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words);
+      hipLaunchKernelGGL(hbm_stream_kernel<1>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words, block_table, chunks_per_block);
       break;
     case 2:
-      hipLaunchKernelGGL(hbm_stream_kernel<2>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words);
+      hipLaunchKernelGGL(hbm_stream_kernel<2>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words, block_table, chunks_per_block);
       break;
     case 4:
-      hipLaunchKernelGGL(hbm_stream_kernel<4>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words);
+      hipLaunchKernelGGL(hbm_stream_kernel<4>, grid, block, 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, words, block_table, chunks_per_block);
       break;
     default:
       return fail(DCP_ERR_UNSUPPORTED, "hbm_stream_probe: n_streams %d unsupported (1, 2 or 4)", n_streams);

@@ -1,31 +1,32 @@
 // Block gather/scatter kernels: pointer-table block copy, per-token dKV copy
 // and head-strided LSE copy.  Pure byte movement, HBM-bound.
 //
-// One workgroup of 256 lanes moves one chunk of one block with 16-byte
-// non-temporal loads and stores; consecutive lanes touch consecutive 16-byte
-// words.  The chunk is 4 KiB (one load per lane) for blocks of 2 MiB and more
-// and 16 KiB (four independent loads per lane) for smaller blocks: measured on
-// a seeded permutation of a 2 GiB bf16 tensor, 4 MiB blocks move at 6.2 TB/s
-// with 4 KiB chunks against 5.8 with 16 KiB, while the 1 MiB / 0.5 MiB blocks
-// of an executor gather take 0.31 ms per launch with 4 KiB chunks against 0.23
-// with 16 KiB.
+// One workgroup moves one chunk of one block with 16-byte non-temporal loads
+// and stores; consecutive lanes touch consecutive 16-byte words.  The chunk is
+// 1 KiB (a single wave, one load per lane) for blocks of 2 MiB and more and for
+// blocks of at most 256 KiB, and 16 KiB (256 lanes, four independent loads per
+// lane) in between: measured on a seeded permutation of a 2 GiB bf16 tensor,
+// 4 MiB blocks move at 6.67 TB/s in 1 KiB chunks, 6.2 in 4 KiB chunks of 256
+// lanes and 5.8 in 16 KiB chunks, while the 1 MiB / 0.5 MiB blocks of an
+// executor gather (ragged, two sizes in one launch) take 0.31 ms per launch
+// with 4 KiB chunks against 0.23 with 16 KiB.
 #include "common.h"
 
 namespace dcp {
 
-constexpr int kCopyThreads = 256;
 // Chunk size by block size, measured on 2 GiB moved through a seeded block permutation: 4 MiB blocks
-// 6.2 TB/s in 4 KiB chunks; 128 KiB blocks 5.7 TB/s in 4 KiB chunks against 5.4 in 16 KiB chunks; the
-// 0.5-1 MiB blocks of an attention plan, ragged and of two sizes in one launch, 6.1 TB/s in 16 KiB
-// chunks against 4.3 in 4 KiB chunks (four times the workgroups that find nothing to move).
-constexpr int64_t kSmallChunkBlockBytes = 2 << 20;   // blocks at least this large use 4 KiB chunks,
+// 6.67 TB/s in 1 KiB chunks (6.2 in 4 KiB chunks); 128 KiB blocks 6.10 TB/s in 1 KiB chunks against 5.88
+// in 4 KiB and 5.4 in 16 KiB chunks; the 0.5-1 MiB blocks of an attention plan, ragged and of two sizes
+// in one launch, 6.1 TB/s in 16 KiB chunks against 4.3 in 4 KiB chunks (four times the workgroups
+// that find nothing to move).
+constexpr int64_t kSmallChunkBlockBytes = 2 << 20;   // blocks at least this large use 1 KiB chunks,
 constexpr int64_t kTinyBlockBytes = 256 << 10;       // and so do blocks at most this large
 
 // Tables are nullable where the dKV variant has no such column: a null
 // offset/stride table means offset 0, and n_count[p] is multiplied by
 // `elems_per_count` (1 for the element-count variant, per_token_size for the
 // token-count variant).
-template <int kCopyUnroll>
+template <int kCopyUnroll, int kCopyThreads>
 __global__ __launch_bounds__(kCopyThreads) void copy_varlen_kernel(
     const int64_t* __restrict__ src_ptrs, const int32_t* __restrict__ src_offsets,
     const int32_t* __restrict__ src_strides, const int64_t* __restrict__ dst_ptrs,
@@ -109,17 +110,18 @@ static int launch_copy(const int64_t* src_ptrs, const int32_t* src_offsets,
                        int64_t block_numel, int elem_size, void* stream) {
   const int64_t block_bytes = block_numel * elem_size;
   const int unroll = block_bytes >= kSmallChunkBlockBytes || block_bytes <= kTinyBlockBytes ? 1 : 4;
-  const int64_t chunk_bytes = (int64_t)kCopyThreads * 16 * unroll;
+  const int threads = unroll == 1 ? 64 : 256;
+  const int64_t chunk_bytes = (int64_t)threads * 16 * unroll;
   const int64_t chunks = (block_bytes + chunk_bytes - 1) / chunk_bytes;
   DCP_REQUIRE(chunks * n_ptrs < (int64_t)1 << 31, "copy grid too large: %lld blocks x %lld chunks",
               (long long)n_ptrs, (long long)chunks);
   KernelTimer timer("copy_varlen_kernel", stream);
   if (unroll == 1)
-    hipLaunchKernelGGL(copy_varlen_kernel<1>, dim3((unsigned)(chunks * n_ptrs)), dim3(kCopyThreads), 0,
+    hipLaunchKernelGGL((copy_varlen_kernel<1, 64>), dim3((unsigned)(chunks * n_ptrs)), dim3(64), 0,
                        (hipStream_t)stream, src_ptrs, src_offsets, src_strides, dst_ptrs,
                        dst_offsets, dst_strides, n_count, elems_per_count, (int)chunks, elem_size);
   else
-    hipLaunchKernelGGL(copy_varlen_kernel<4>, dim3((unsigned)(chunks * n_ptrs)), dim3(kCopyThreads), 0,
+    hipLaunchKernelGGL((copy_varlen_kernel<4, 256>), dim3((unsigned)(chunks * n_ptrs)), dim3(256), 0,
                        (hipStream_t)stream, src_ptrs, src_offsets, src_strides, dst_ptrs,
                        dst_offsets, dst_strides, n_count, elems_per_count, (int)chunks, elem_size);
   return check_launch("copy_varlen_kernel");

@@ -118,7 +118,7 @@ def test_fused_copy_lse_bit_exact(gpu, heads):
 
 
 def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, inf_frac=0.0,
-                unpadded=True, nan_frac=0.0):
+                unpadded=True, nan_frac=0.0, min_width=1, raw=None):
     from dcp_amd.ops.fused_ops import flash_attn_update_out_lse
 
     g = torch.Generator().manual_seed(seed)
@@ -136,7 +136,7 @@ def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, in
     if nan_frac > 0:
         src_lse[torch.rand(src_lse.shape, generator=g) < nan_frac] = float("nan")
     blocks = rng.permutation(n_src_blocks)[: sum(n_src_per_op)]
-    width = 1 << (max(n_src_per_op) - 1).bit_length()
+    width = max(min_width, 1 << (max(n_src_per_op) - 1).bit_length())
     table, c = [], 0
     for n in n_src_per_op:
         table.append(list(blocks[c : c + n]) + [-1] * (width - n))
@@ -170,6 +170,8 @@ def _merge_case(gpu, dtype, n_src_per_op, n_head, head_dim, block_size, seed, in
         i32(n_src_per_op), block_size, block_size * n_head * head_dim, n_head * head_dim, block_size, 1,
         n_src_blocks * block_size, dst_head_stride, head_dim, width, 64)
     torch.cuda.synchronize()
+    if raw is not None:  # the caller compares bit patterns between launches
+        raw.append((d_dst_out.cpu(), d_dst_lse.cpu()))
     got_out = d_dst_out.float().cpu().numpy().reshape(-1, n_head, head_dim)
     got_lse = d_dst_lse.cpu().numpy().reshape(n_head, -1)
     max_out = max_lse = 0.0
@@ -226,6 +228,25 @@ def test_update_out_lse_wide_rows(gpu, name, tol):
     assert err_out <= tol and err_lse <= 1e-3, (err_out, err_lse)
     err_out, err_lse = _merge_case(gpu, dtype, [2, 2, 3], heads, 128, 128, seed=6, unpadded=False)
     assert err_out <= tol and err_lse <= 1e-3, (err_out, err_lse)
+
+
+@pytest.mark.parametrize("name,tol", [("fp32", 2e-5), ("bf16", 2e-2), ("fp16", 4e-3)])
+def test_update_out_lse_wide_rows_of_few_sources(gpu, name, tol):
+    """Launches whose ops have at most four sources take the one-wave kernel on wide rows (the
+    lanes of a quad share the exponentials): ragged token counts, ignored and NaN sources, tables
+    of width 4, 2 and 1, unpadded destination; and the same ops through a table padded to eight
+    columns (the workgroup kernel with its weights in LDS) give the same bits."""
+    dtype = DTYPES[name]
+    heads = 16 if name != "fp32" else 8
+    bits = lambda t: t.view(torch.int16 if t.element_size() == 2 else torch.int32)
+    # (NaN LSEs only where every op has two sources or more: a single-source op copies bits)
+    for sources, seed, nan_frac in (([2, 4, 3, 4], 21, 0.01), ([2, 4, 1, 3], 24, 0.0), ([2, 1, 2], 22, 0.0), ([1, 1], 23, 0.0)):
+        raw = []
+        for min_width in (1, 8):
+            err_out, err_lse = _merge_case(gpu, dtype, sources, heads, 128, 64, seed=seed, inf_frac=0.3, nan_frac=nan_frac,
+                                           min_width=min_width, raw=raw)
+            assert err_out <= tol and err_lse <= 1e-3, (sources, min_width, err_out, err_lse)
+        assert torch.equal(bits(raw[0][0]), bits(raw[1][0])) and torch.equal(bits(raw[0][1]), bits(raw[1][1])), sources
 
 
 def test_update_out_lse_single_source_is_exact_copy(gpu):
@@ -365,14 +386,25 @@ def test_roofline_probes(gpu):
     src = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=4 * per_stream // 4, dtype=np.int64).astype(np.int32)).to(gpu)
     dst = torch.zeros(per_stream // 4, dtype=torch.int32, device=gpu)
     for n in (1, 2, 4):
-        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), n, per_stream, stream)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), n, per_stream, None, 0, stream)
         torch.cuda.synchronize()
         want = src.reshape(4, -1)[:n].to(torch.int64).sum(0).to(torch.int32)  # wraps like the 32-bit adds
         assert torch.equal(dst, want), n
+    # streams made of 2 KiB blocks picked from `src` through a table: block b of stream s = table[b][s]
+    block_bytes, n_blocks = 2048, per_stream // 2048
+    for n in (1, 4):
+        table = torch.from_numpy(rng.permutation(4 * n_blocks)[: n * n_blocks].reshape(n_blocks, n).astype(np.int32)).to(gpu)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), n, per_stream, table.data_ptr(), block_bytes, stream)
+        torch.cuda.synchronize()
+        blocks = src.reshape(4 * n_blocks, block_bytes // 4).to(torch.int64)
+        want = blocks[table.long()].sum(1).to(torch.int32).reshape(-1)
+        assert torch.equal(dst, want), n
     with pytest.raises(ValueError):
-        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 3, per_stream, stream)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 3, per_stream, None, 0, stream)
     with pytest.raises(AssertionError):
-        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 1, 100, stream)
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 1, 100, None, 0, stream)
+    with pytest.raises(AssertionError):
+        call_probe("bench_hbm_stream_probe", src.data_ptr(), dst.data_ptr(), 1, per_stream, dst.data_ptr(), 3000, stream)
 
     n_wg, iters = 8, 10
     ops = torch.full((n_wg * 256 * 16 * 8,), 0.5, device=gpu, dtype=torch.bfloat16)
