@@ -341,14 +341,22 @@ def movement_microbench(iters=5, bs=512):
     fused_copy_bf16_varlen(*scatter1, numel1, 128)
     torch.cuda.synchronize()
     exact = exact and bool(torch.equal(back, src))
-    _lib.profile_enable(True)
-    for _ in range(iters):
+    # every launch timed by itself (events on the launch stream): the first launches after another
+    # kernel's working set run slower than the ones that follow, so both rates are reported
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(2 * max(iters, 8) + 1)]
+    marks[0].record()
+    for i in range(max(iters, 8)):
         fused_copy_bf16_varlen(*gather1, numel1, 128)
+        marks[2 * i + 1].record()
         fused_copy_bf16_varlen(*scatter1, numel1, 128)
+        marks[2 * i + 2].record()
     torch.cuda.synchronize()
-    _lib.profile_enable(False)
-    n, total = _lib.profile_report()["copy_varlen_kernel"]
-    copy1_gbps = copy_bytes / (total / n * 1e-3) / 1e9
+    launch_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(len(marks) - 1)]
+    one_launch_bytes = copy_bytes / 2
+    copy1_gbps = one_launch_bytes / (sum(launch_ms) / len(launch_ms) * 1e-3) / 1e9
+    copy1_first_gbps = one_launch_bytes / (sum(launch_ms[:4]) / 4 * 1e-3) / 1e9
+    steady = sorted(launch_ms[4:])
+    copy1_steady_gbps = one_launch_bytes / (steady[len(steady) // 2] * 1e-3) / 1e9
     del packed, back
 
     # merge: 4 partial outs per q block
@@ -408,6 +416,9 @@ def movement_microbench(iters=5, bs=512):
         gather_scatter_GBps=round(copy_gbps, 1),
         gather_scatter_frac_of_8TBps=round(copy_gbps / PEAK_HBM_GBPS, 4),
         gather_scatter_one_head_blocks_GBps=round(copy1_gbps, 1),
+        gather_scatter_one_head_blocks_first_4_launches_GBps=round(copy1_first_gbps, 1),
+        gather_scatter_one_head_blocks_steady_GBps=round(copy1_steady_gbps, 1),
+        gather_scatter_one_head_blocks_steady_frac_of_8TBps=round(copy1_steady_gbps / PEAK_HBM_GBPS, 4),
         gather_scatter_roundtrip_bit_exact=exact,
         copy_bytes_per_launch=copy_bytes,
         merge4_GBps=round(merge_gbps, 1),

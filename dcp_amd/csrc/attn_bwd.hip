@@ -253,9 +253,16 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     load_async_dword(at + sc_at_second, voff, base + sc_second_bytes);
   };
 
-  // dS pieces (WRITE_DS): number of this wave's 64-key half tile among all rows' (the rows' key
-  // counts are multiples of 64), and the lane's 16 bytes within a [key][query half] plane of a piece
-  const int64_t ds_tile64 = (int64_t)(p.cu_seqlens_kv[b] / 64) + 2 * kt + (w >> 1);
+  // dS pieces (WRITE_DS).  The workspace holds the rows one after another; row b starts at 64-key
+  // tile cu_seqlens_kv[b] / 64 + b (room for a last, partial tile of every row before it) and is laid
+  // out [head][32-query chunk][64-key tile]: the pieces that a wave of the dQ kernel reads one after
+  // another lie one after another (ordered by key tile first, they were 4 MiB apart at 32 heads and
+  // 1024-token blocks, every one in a memory page of its own).  ds_lane: the lane's 16 bytes within a
+  // [key][query half] plane of a piece.
+  const int ds_row_tiles = (seqlen_kv + 63) / 64;
+  const uint64_t ds_row_base = ((uint64_t)(p.cu_seqlens_kv[b] / 64) + b) * p.n_heads_q * p.subs_per_row;
+  const int ds_tile_local = 2 * kt + (w >> 1);
+  const uint64_t ds_chunk_bytes = has_keys ? (uint64_t)ds_row_tiles << 12 : 4096;  // from a 32-query chunk to the next
   const int ds_lane = (w & 1) * 128 + 2 * c + h;
 
   // steps: (q head of the group) x (active 64-query tile)
@@ -308,10 +315,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
     // (a wave whose 32 keys lie past the row's last key has no piece -- its 64-key half tile would be
     // the next row's first, or lie past the end of the workspace -- and writes its zeros into two
     // spare pieces behind the last one instead: no branch around the stores)
-    const uint64_t ds_step = WRITE_DS ? uniform64(reinterpret_cast<uint64_t>(p.ds) +
-                                                  (((has_keys ? ((uint64_t)ds_tile64 * p.n_heads_q + (kv_head * group + hg)) * p.subs_per_row + 2 * qt
-                                                              : (uint64_t)p.ds_pieces)) << 12))
-                                      : 0;
+    const uint64_t ds_step =
+        WRITE_DS ? uniform64(reinterpret_cast<uint64_t>(p.ds) +
+                             (((has_keys ? ds_row_base + ((uint64_t)(kv_head * group + hg) * p.subs_per_row + 2 * qt) * ds_row_tiles + ds_tile_local
+                                         : (uint64_t)p.ds_pieces))
+                              << 12))
+                 : 0;
 
     // One sub-step = this wave's 32 keys against 32 of the step's 64 queries (QI = 0, 1).
     // (A real loop, not unrolled: one copy of the body keeps the register allocation of a single
@@ -431,7 +440,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dkv_kernel(const Attn
         // (below), like the tile loads of the first.
       }
       typedef __attribute__((address_space(1))) u32x4 global_u32x4;
-      global_u32x4* piece = (global_u32x4*)(ds_step + ((uint64_t)QI << 12)) + ds_lane;
+      global_u32x4* piece = (global_u32x4*)(ds_step + (uint64_t)QI * ds_chunk_bytes) + ds_lane;
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(kPrioMatrix);
 #pragma unroll
@@ -898,7 +907,7 @@ static int attn_bwd_launch(const void* dout, const void* q, const void* k, const
   const bool fused = allow_fused && head_dim == 128 && bwd_fused_available() && workspace_bytes >= base + extra;
   // The backward through dS in memory where it is selected, the caller said how many keys the rows
   // have in all and the workspace holds the dS pieces.
-  const size_t ds_bytes = bwd_ds_workspace_bytes(total_kv, block_size, n_heads_q);
+  const size_t ds_bytes = bwd_ds_workspace_bytes(total_kv, batch, block_size, n_heads_q);
   const bool through_ds = allow_fused && !fused && bwd_select(-1) == DCP_BWD_THROUGH_DS && total_kv > 0 &&
                           workspace_bytes >= base + ds_bytes;
   DCP_REQUIRE(workspace_bytes >= base, "attn_bwd: workspace of %zu bytes is smaller than the %zu needed",
@@ -1030,7 +1039,7 @@ extern "C" size_t dcp_attn_bwd_workspace_bytes_kv(int batch, int total_q, int64_
                                                   int n_heads_q, int head_dim) {
   const size_t base = dcp_attn_bwd_workspace_bytes(batch, total_q, block_size, n_heads_q, head_dim);
   if (base == 0 || bwd_select(-1) != DCP_BWD_THROUGH_DS) return base;
-  return base + bwd_ds_workspace_bytes(total_kv, block_size, n_heads_q);
+  return base + bwd_ds_workspace_bytes(total_kv, batch, block_size, n_heads_q);
 }
 
 // ---------------------------------------------------------------------------

@@ -17,8 +17,19 @@
 // in whole 1 KiB stores.  A wave here owns 32 queries (one piece per 64-key tile), brings its
 // pieces into a region of LDS of its own with global_load_lds and reads them as the B operand
 // through transposing loads, whose per-lane addresses undo the layout; no other wave touches the
-// piece, so it needs no barrier, only the wave's own wait.  K tiles are shared by the four waves
-// as in the other kernels.
+// piece, so it needs no barrier, only the wave's own wait.  K tiles are shared by the workgroup's
+// waves as in the other kernels.
+//
+// The kernel does nothing but wait for memory unless loads are in flight all the time (with the
+// matrix instructions taken out it runs as long as with them, and with the K loads or the barriers
+// taken out too), so a workgroup is eight waves (256 queries, one workgroup per CU: half the K traffic
+// of four-wave workgroups) with three stages of K tile and pieces in LDS: while tile t is multiplied,
+// the loads of tiles t + 1 and t + 2 are under way, and a wave waits for tile t alone by counting
+// its own loads (vmcnt), not for everything.  On the 65536-token causal benchmark (16.8 GB of dS) it
+// takes 3.2 ms, 5.5 TB/s out of HBM, against 3.4 ms for four-wave workgroups with two stages and
+// a full wait per tile; a kernel that only streams 4 KiB pieces per wave into LDS the same way
+// reads 7.0 TB/s, and what is left between the two is the start of every work item (a chain of
+// dependent table reads and an empty pipeline, about 35 times per workgroup).
 #include <math.h>
 
 #include <algorithm>
@@ -27,17 +38,19 @@
 
 namespace dcp {
 
-constexpr int kDsBM = 128;  // queries per workgroup
-constexpr int kDsBN = 64;   // keys per tile
+constexpr int kDsWaves = 8;
+constexpr int kDsThreads = 64 * kDsWaves;
+constexpr int kDsBM = 32 * kDsWaves;  // queries per workgroup
+constexpr int kDsBN = 64;             // keys per tile
+constexpr int kDsStages = 3;
 
 template <int DTYPE, int D>
 __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, int item) {
   constexpr int BN = kDsBN;
   constexpr int DT = D / 32;
-  typedef KvTile<D> Tile;
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds0[Tile::SIZE];
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds1[Tile::SIZE];
-  __shared__ __attribute__((aligned(16))) uint16_t ds_lds[2][4][2048];  // [stage][wave]: one piece
+  typedef KvTile<D, kDsWaves> Tile;
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[kDsStages][Tile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t ds_lds[kDsStages][kDsWaves][2048];  // [stage][wave]: one piece
   __shared__ int slot_lds[kSlotTableCap];
 
   const int tid = threadIdx.x;
@@ -65,7 +78,8 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   // ---- which key tiles: the 128-key tiles the dK/dV kernel visited for this wave's 64-query tile
   // (the same test on the same hulls: a piece that was never written is never read), and for the
   // workgroup the hull of its two 64-query tiles -----------------------------------------------
-  const int qt64 = 2 * qt + (w >> 1);
+  constexpr int T64 = kDsBM / 64;  // 64-query tiles of a workgroup
+  const int qt64 = T64 * qt + (w >> 1);
   const bool wave_has_tile = qt64 < p.q_tiles_per_row;
   const int32_t* hull_row = p.hull + (int64_t)b * p.q_tiles_per_row * 8;
   int hw[4] = {0x7fffffff, 0, 0x7fffffff, 0};
@@ -76,9 +90,9 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   const TileRuns mine(hw[0], hw[1], hw[2], hw[3], 128);  // in 128-key tiles
   int g[4] = {0x7fffffff, 0, 0x7fffffff, 0};
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    if (2 * qt + t >= p.q_tiles_per_row) continue;
-    const int32_t* hu = hull_row + (2 * qt + t) * 8;
+  for (int t = 0; t < T64; ++t) {
+    if (T64 * qt + t >= p.q_tiles_per_row) continue;
+    const int32_t* hu = hull_row + (T64 * qt + t) * 8;
     g[0] = min(g[0], __builtin_amdgcn_readfirstlane(hu[0]));
     g[1] = max(g[1], __builtin_amdgcn_readfirstlane(hu[1]));
     g[2] = min(g[2], __builtin_amdgcn_readfirstlane(hu[2]));
@@ -96,7 +110,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   const int n_tiles = runs.count();
 
   const int32_t* kv_table = p.kv_block_table + (int64_t)b * p.max_kv_blocks;
-  load_slot_table(slot_lds, kv_table, p.max_kv_blocks, tid, kBwdThreads);
+  load_slot_table(slot_lds, kv_table, p.max_kv_blocks, tid, kDsThreads);
   __syncthreads();
 
   f32x16 dq_acc[DT];
@@ -117,11 +131,13 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   const int tiles_per_block = p.block_size / BN;
   const int64_t tile_stride = (int64_t)BN * p.kv_token_stride;
   TileCursor cursor;
-  // the wave's piece of key tile t: ((first 64-key tile of the row + t) * heads + head) * sub-tiles + sub-tile
-  const int sub = qt * 4 + w;
+  // the wave's piece of key tile t (the layout is described in the dK/dV kernel): its pieces lie one
+  // after another in key order
+  const int sub = qt * kDsWaves + w;
+  const uint64_t row_base = ((uint64_t)(kv_begin / 64) + b) * p.n_heads_q * p.subs_per_row;
   const uint64_t piece0 = reinterpret_cast<uint64_t>(p.ds) +
-                          ((((uint64_t)(kv_begin / 64) * p.n_heads_q + head) * p.subs_per_row + sub) << 12);
-  const uint64_t piece_step = ((uint64_t)p.n_heads_q * p.subs_per_row) << 12;
+                          ((row_base + ((uint64_t)head * p.subs_per_row + sub) * (uint64_t)last64) << 12);
+  const uint64_t piece_step = 4096;
   auto wave_sees = [&](int t64) {
     const int t = t64 >> 1;
     return wave_has_tile && ((t >= mine.a0 && t < mine.b0) || (t >= mine.a1 && t < mine.b1));
@@ -171,34 +187,38 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
     }
   };
 
-  const uint32_t k_at0 = lds_address(k_lds0), k_at1 = lds_address(k_lds1);
-  const uint32_t ds_at0 = lds_address(&ds_lds[0][w][0]), ds_at1 = lds_address(&ds_lds[1][w][0]);
+  // Stage s holds tile i with i % kDsStages == s.  Before it multiplies tile i, a wave waits until
+  // the loads it issued for tile i have landed -- the ones for tile i + 1, issued after them, may
+  // still be under way: vmcnt counts a wave's loads in order -- and meets the others at a barrier:
+  // everybody's share of K tile i is there, and everybody is done with tile i - 1, whose stage
+  // the loads of tile i + 2 now refill.
+  const uint32_t k_at0 = lds_address(&k_lds[0][0]), ds_at0 = lds_address(&ds_lds[0][w][0]);
+  constexpr uint32_t kKStageBytes = Tile::SIZE * 2, kDsStageBytes = kDsWaves * 4096;
+  auto request_into = [&](int stage) {
+    fill_k = k_at0 + stage * kKStageBytes;
+    fill_ds = ds_at0 + stage * kDsStageBytes;
+    request();
+  };
   if (n_tiles > 0) {
     cursor.seek(runs, 0, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
-    fill_k = k_at0;
-    fill_ds = ds_at0;
-    request();
-  }
-  for (int i = 0; i < n_tiles; i += 2) {
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // stage 0 is filled; nobody reads stage 1 any more
-    if (i + 1 < n_tiles) {
+    request_into(0);
+    if (n_tiles > 1) {
       advance();
-      fill_k = k_at1;
-      fill_ds = ds_at1;
-      request();
+      request_into(1);
     }
-    compute(runs.tile(i), k_lds0, &ds_lds[0][w][0]);
-    if (i + 1 >= n_tiles) break;
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // stage 1 is filled; nobody reads stage 0 any more
+  }
+  int stage = 0;
+  for (int i = 0; i < n_tiles; ++i) {
+    if (i + 1 >= n_tiles) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (wave_sees(runs.tile(i + 1))) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL + 4) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+    phase_barrier();
     if (i + 2 < n_tiles) {
       advance();
-      fill_k = k_at0;
-      fill_ds = ds_at0;
-      request();
+      request_into(stage == 0 ? 2 : stage - 1);  // (i + 2) % 3
     }
-    compute(runs.tile(i + 1), k_lds1, &ds_lds[1][w][0]);
+    compute(runs.tile(i), &k_lds[stage][0], &ds_lds[stage][w][0]);
+    stage = stage == kDsStages - 1 ? 0 : stage + 1;
   }
 
   if (!q_valid) return;
@@ -216,7 +236,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
 
 // persistent, like the recomputing dQ kernel: per-XCD tickets in the workspace (zeroed by the prepare kernel)
 template <int DTYPE, int D>
-__global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_ds_kernel(const AttnBwdParams p) {
+__global__ __launch_bounds__(kDsThreads, 1) void attn_bwd_dq_ds_kernel(const AttnBwdParams p) {
   __shared__ int ticket_lds;
   const int x = blockIdx.x % kNumXcd;
   const int64_t n_streams = (p.n_dq_items + p.dq_xcd_group - 1) / p.dq_xcd_group;
@@ -232,25 +252,31 @@ __global__ __launch_bounds__(kBwdThreads, 2) void attn_bwd_dq_ds_kernel(const At
   }
 }
 
-size_t bwd_ds_workspace_bytes(int64_t total_kv, int block_size, int n_heads_q) {
+size_t bwd_ds_workspace_bytes(int64_t total_kv, int batch, int block_size, int n_heads_q) {
   if (total_kv <= 0) return 0;
   const size_t subs = (block_size + 31) / 32;
-  return ((size_t)((total_kv + 63) / 64) * n_heads_q * subs + 2) << 12;  // and two spare pieces (see the dK/dV kernel)
+  // a 64-key tile more per row than total_kv / 64 (rows may end inside a tile), and two spare pieces (see the dK/dV kernel)
+  return ((size_t)(total_kv / 64 + batch + 1) * n_heads_q * subs + 2) << 12;
 }
 
 int launch_bwd_through_ds(const AttnBwdParams& p, int dtype, hipStream_t stream) {
   if (const int e = launch_bwd_prepare(p, dtype, stream)) return e;  // (also zeroes the dQ kernel's tickets)
   if (const int e = launch_bwd_dkv_writing_ds(p, dtype, stream)) return e;
-  const int64_t n_dq = std::min<int64_t>(xcd_grid_size(p.n_dq_items, 1), xcd_grid_size(2 * (int64_t)device_cu_count(), 1));
-  DCP_REQUIRE(p.n_dq_items < ((int64_t)1 << 31), "attn_bwd: grid too large");
+  // this dQ kernel's work items: (row, head, 256-query tile); the tiles and heads that share a K stay on one XCD
+  AttnBwdParams q = p;
+  q.dq_tiles_per_row = (p.block_size + kDsBM - 1) / kDsBM;
+  q.n_dq_items = (int64_t)p.batch * p.n_heads_q * q.dq_tiles_per_row;
+  q.dq_xcd_group = q.dq_tiles_per_row * (p.n_heads_q / p.n_heads_kv);
+  DCP_REQUIRE(q.n_dq_items < ((int64_t)1 << 31), "attn_bwd: grid too large");
+  const int64_t n_dq = std::min<int64_t>(xcd_grid_size(q.n_dq_items, 1), xcd_grid_size((int64_t)device_cu_count(), 1));
   KernelTimer timer("attn_bwd_dq_ds_kernel", stream);
-  const dim3 grid((unsigned)n_dq), block(kBwdThreads);
+  const dim3 grid((unsigned)n_dq), block(kDsThreads);
   if (dtype == DCP_DTYPE_BF16) {
-    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_BF16, 128>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_BF16, 64>), grid, block, 0, stream, p);
+    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_BF16, 128>), grid, block, 0, stream, q);
+    else hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_BF16, 64>), grid, block, 0, stream, q);
   } else {
-    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_FP16, 128>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_FP16, 64>), grid, block, 0, stream, p);
+    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_FP16, 128>), grid, block, 0, stream, q);
+    else hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_FP16, 64>), grid, block, 0, stream, q);
   }
   return check_launch("attn_bwd_dq_ds_kernel");
 }

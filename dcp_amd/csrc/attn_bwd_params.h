@@ -82,7 +82,7 @@ constexpr int kTicketInts = 16;  // one counter per XCD (the rest unused)
 int launch_bwd_through_ds(const AttnBwdParams& p, int dtype, hipStream_t stream);
 int launch_bwd_prepare(const AttnBwdParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dkv_writing_ds(const AttnBwdParams& p, int dtype, hipStream_t stream);
-size_t bwd_ds_workspace_bytes(int64_t total_kv, int block_size, int n_heads_q);
+size_t bwd_ds_workspace_bytes(int64_t total_kv, int batch, int block_size, int n_heads_q);
 
 // The one-pass backward (prepare + fused kernel) for head size 128; p.hull, p.delta, p.lse2,
 // p.dq_part, p.chain and p.fault point into the workspace.
