@@ -38,9 +38,11 @@ class SymbolicDevice:
         # so that a read of recycled contents can say what happened and the run can report reuse
         self.history = defaultdict(list)  # (buffer type, index) -> [name, ...]
         self.overwritten = 0              # writes that replaced contents of another block
+        self.reads = defaultdict(int)     # (buffer type, index) -> reads of the present contents
 
     def get(self, block):
         assert block.index < len(self.slots[block.buffer_type]), f"{block} outside its buffer"
+        self.reads[(block.buffer_type, block.index)] += 1
         return self.slots[block.buffer_type][block.index]
 
     def expect(self, block, name):
@@ -58,6 +60,15 @@ class SymbolicDevice:
         old = self.slots[block.buffer_type][block.index]
         if old is not None and old[:4] != name[:4]:
             self.overwritten += 1
+            # An input block (a gathered or received Q, KV, OUT, LSE or dOUT block) is put into a slot
+            # for some instruction to read.  Replaced before anything has read it, its slot was given
+            # away too early: the instruction it was meant for will find the newcomer (which a check
+            # of what that instruction reads cannot tell when the newcomer looks just as plausible).
+            if old[0] in _LOCAL_INPUTS.values() and block.buffer_type.startswith("Buffer"):
+                assert self.reads[(block.buffer_type, block.index)] > 0, (
+                    f"{block}: {old} is overwritten by {name} before any instruction read it "
+                    f"(slot history {self.history[(block.buffer_type, block.index)]})")
+        self.reads[(block.buffer_type, block.index)] = 0
         self.history[(block.buffer_type, block.index)].append(name)
         self.slots[block.buffer_type][block.index] = name
 
@@ -102,7 +113,6 @@ def _attention(dev, instr, group_of, backward):
         assert q[0] == "Q"
         _, g, s, i = q
         kv_ids = []
-        dev.expect(q_block, q)
         assert instr.seqlens_kv[b] == bs * len(instr.kv_block_table[b])
         for kv_block in instr.kv_block_table[b]:
             assert kv_block.buffer_type == "BufferKV"

@@ -97,6 +97,60 @@ def test_the_checker_notices_a_slot_recycled_too_early():
         run_symbolic(plans, case["layouts"], case["n_devices_per_node"], False, case["mask"], _q_per_kv(cfg))
 
 
+def test_the_checker_notices_an_input_slot_given_away_before_its_block_was_read():
+    """A receive redirected into a slot whose block (received or gathered earlier) no stage has read
+    yet -- its first reader runs after the redirected receive completes: the block is replaced before
+    anything has read it, and the checker says so at the write.  (What the later stage then finds may
+    look plausible, so the read itself need not fail.)"""
+    cfg = MULTI["staged_four_stages"]
+    case = make_multi_case(**cfg)
+    plans = case["fw"]
+
+    def redirect_one(plan):
+        ins = plan.instructions
+        wait_at = {i.key: j for j, i in enumerate(ins) if type(i).__name__ == "CommWaitInstr"}
+        writes, reads = {}, {}  # slot -> [(time, n_tokens)], slot -> [time]
+        for j, i in enumerate(ins):
+            if type(i).__name__ == "MemcpyInstr":
+                for _, dst in i.src_dst_pairs:
+                    writes.setdefault((dst.buffer_type, dst.index), []).append((j, dst.n_tokens))
+            elif isinstance(i, CommLaunchInstr):
+                for op in i.comm_ops:
+                    if op.comm_type == 1:
+                        blk = op.buffer_block
+                        writes.setdefault((blk.buffer_type, blk.index), []).append((wait_at[i.key], blk.n_tokens))
+            elif type(i).__name__ == "AttnInstr":
+                for row in i.q_block_table:
+                    reads.setdefault((row[0].buffer_type, row[0].index), []).append(j)
+                for row in i.kv_block_table:
+                    for blk in row:
+                        reads.setdefault((blk.buffer_type, blk.index), []).append(j)
+        for launch in (i for i in ins if isinstance(i, CommLaunchInstr)):
+            w2 = wait_at[launch.key]
+            for k, op in enumerate(launch.comm_ops):
+                blk = op.buffer_block
+                if op.comm_type != 1 or blk.buffer_type not in ("BufferQ", "BufferKV"):
+                    continue
+                for slot, ws in writes.items():
+                    if slot[0] != blk.buffer_type or slot[1] == blk.index:
+                        continue
+                    before = [(t, n) for t, n in ws if t < w2]
+                    if not before or before[-1][1] != blk.n_tokens:
+                        continue
+                    w1 = before[-1][0]
+                    rs = reads.get(slot, [])
+                    if any(w1 < r < w2 for r in rs) or not any(r > w2 for r in rs):
+                        continue  # already read, or nobody waits for it
+                    launch.comm_ops[k] = CommOp(op.comm_type, op.peer, BufferBlock(slot[0], slot[1], blk.n_tokens))
+                    return True
+        return False
+
+    if not any(redirect_one(plan) for plan in plans):
+        pytest.skip("no device of this case holds an unread input block while a receive completes")
+    with pytest.raises(AssertionError, match="before any instruction read it"):
+        run_symbolic(plans, case["layouts"], case["n_devices_per_node"], False, case["mask"], _q_per_kv(cfg))
+
+
 def test_the_checker_notices_a_wrong_plan():
     """A kv block swapped in an attention row, a receive into the wrong kind of slot and a dropped
     work unit must each fail."""
