@@ -122,6 +122,12 @@ class AttentionExecutor(DCPExecutor):
         self._barrier_generation: Dict[int, int] = {}
         self.n_heads_per_block = n_heads_per_block
         self.head_dim = head_dim
+        # The kernels exist for head sizes 64 and 128.  Another head size (up to 128) is stored at the
+        # next of the two in every buffer this executor owns, the added columns zero (zero q and k
+        # columns leave the scores unchanged; zero v and dout columns give zero out, dq, dk, dv
+        # columns), so that no call pads or copies anything: the reference pads head sizes to what
+        # its kernels take, too (dcp/runtime/flash_attention/executor.py:156-160).
+        self.kernel_head_dim = head_dim if head_dim is None or head_dim > 128 else (64 if head_dim <= 64 else 128)
         self.main_stream = torch.cuda.Stream()
         self.streams: Dict[str, torch.cuda.Stream] = {}
         self._prep_handlers = HandlerTable("Prep handler")
@@ -143,17 +149,42 @@ class AttentionExecutor(DCPExecutor):
         return torch.zeros(*buffer_shape, dtype=int_to_torch_dtype(buffer_dtype), device="cuda")
 
     def init_buffers(self, execution_plan: ExecutionPlan):
-        """As the base class, but the unpadded token-major tensors get one block of zeroed tokens
-        behind their last one: kernels that address them directly load whole tiles, i.e. up to a
-        block past a ragged last block (masked, but it has to be readable and finite)."""
+        """As the base class, with two differences.  The unpadded token-major tensors get one block of
+        zeroed tokens behind their last one: kernels that address them directly load whole tiles,
+        i.e. up to a block past a ragged last block (masked, but it has to be readable and finite).
+        And a head size the kernels do not have is stored at the next one they have (see
+        ``kernel_head_dim``): shapes, per-token sizes and block strides are those of the wider rows."""
+        d, dk = self.head_dim, self.kernel_head_dim
         for buffer_type, info in execution_plan.buffer_info.items():
-            if (self.buffers.get(buffer_type) is None and buffer_type.startswith("Local")
-                    and buffer_type not in _LSE_BUFFER_TYPES and len(info.buffer_shape) >= 2):
-                shape = tuple(info.buffer_shape)
+            shape, per_token_shape, numel = tuple(info.buffer_shape), tuple(info.per_token_shape), info.block_numel
+            if dk != d and buffer_type not in _LSE_BUFFER_TYPES and shape and shape[-1] == d:
+                shape, per_token_shape, numel = shape[:-1] + (dk,), per_token_shape[:-1] + (dk,), numel // d * dk
+            self.buffer_n_blocks[buffer_type] = info.n_blocks
+            self.buffer_block_strides[buffer_type] = numel
+            self.buffer_block_sizes[buffer_type] = info.block_size
+            self.buffer_per_token_shape[buffer_type] = per_token_shape
+            if self.buffers.get(buffer_type) is not None:
+                continue
+            if buffer_type.startswith("Local") and buffer_type not in _LSE_BUFFER_TYPES and len(shape) >= 2:
                 per_token = int(np.prod(shape[1:]))
                 flat = torch.zeros((shape[0] + info.block_size) * per_token, dtype=int_to_torch_dtype(info.dtype), device="cuda")
                 self.buffers[buffer_type] = flat[: shape[0] * per_token].view(shape)
-        super().init_buffers(execution_plan)
+            else:
+                self.buffers[buffer_type] = self._create_buffer(shape, info.dtype)
+
+    def _user_view(self, buffer_type):
+        """The caller's view of a buffer: without the columns added for the kernels' head size."""
+        buf = self.buffers[buffer_type]
+        if self.kernel_head_dim != self.head_dim and buffer_type not in _LSE_BUFFER_TYPES:
+            return buf[..., : self.head_dim]
+        return buf
+
+    def init_forward_input(self, local_q, local_kv):
+        self._user_view(BufferType.LOCAL_Q).copy_(local_q)
+        self._user_view(BufferType.LOCAL_KV).copy_(local_kv)
+
+    def init_backward_input(self, local_dout):
+        self._user_view(BufferType.LOCAL_dOUT).copy_(local_dout)
 
     def log_memory_usage(self):
         total = 0.0
@@ -169,7 +200,7 @@ class AttentionExecutor(DCPExecutor):
         return total
 
     def set_local_out_lse(self, out, lse):
-        self.buffers[BufferType.LOCAL_OUT].copy_(out)
+        self._user_view(BufferType.LOCAL_OUT).copy_(out)
         self.buffers[BufferType.LOCAL_LSE].copy_(lse)
 
     def deallocate_all_buffers(self):
@@ -256,8 +287,8 @@ class AttentionExecutor(DCPExecutor):
         prev_stream.wait_stream(self.main_stream)
         torch.cuda.nvtx.range_pop()
         if is_forward:
-            return self.buffers[BufferType.LOCAL_OUT], self.buffers[BufferType.LOCAL_LSE]
-        return self.buffers[BufferType.LOCAL_dQ], self.buffers[BufferType.LOCAL_dKV]
+            return self._user_view(BufferType.LOCAL_OUT), self.buffers[BufferType.LOCAL_LSE]
+        return self._user_view(BufferType.LOCAL_dQ), self._user_view(BufferType.LOCAL_dKV)
 
     # -- one instruction at a time (several devices' plans run in turns: fabric.execute_together) --
     def begin(self, execution_plan):
@@ -295,7 +326,7 @@ class AttentionExecutor(DCPExecutor):
         self.init_forward_input(q, kv)
         self.execute(self.fw_exec_plan, is_forward=True)
         return (
-            self.buffers[BufferType.LOCAL_OUT].detach().clone(),
+            self._user_view(BufferType.LOCAL_OUT).detach().clone(),
             self.buffers[BufferType.LOCAL_LSE].detach().clone(),
         )
 
@@ -305,8 +336,8 @@ class AttentionExecutor(DCPExecutor):
         self.init_backward_input(dout)
         self.execute(self.bw_exec_plan, is_forward=False)
         return (
-            self.buffers[BufferType.LOCAL_dQ].detach().clone(),
-            self.buffers[BufferType.LOCAL_dKV].detach().clone(),
+            self._user_view(BufferType.LOCAL_dQ).detach().clone(),
+            self._user_view(BufferType.LOCAL_dKV).detach().clone(),
         )
 
 
@@ -675,12 +706,12 @@ def _handle_reduction(exec: AttentionExecutor, instr: AttnReductionInstr):
         n_srcs,
         exec.buffer_block_sizes[src_out_t],
         exec.buffer_block_strides[src_out_t],
-        exec.n_heads_per_block * exec.head_dim,
+        exec.n_heads_per_block * exec.kernel_head_dim,
         exec.buffer_block_sizes[src_lse_t],
         1,
         exec.buffer_n_blocks[src_lse_t] * exec.buffer_block_sizes[src_lse_t],
         dst_lse_head_stride,
-        exec.head_dim,
+        exec.kernel_head_dim,
         width,
         64,
     )

@@ -176,6 +176,27 @@ def test_backward_matches_dense_truth(gpu, name):
     check_against_truth(res, dense_truth(case, backward=True))
 
 
+def test_other_head_sizes_allocate_nothing_per_call(gpu):
+    """The executor stores a head size the kernels do not have at the next one they have, in every
+    buffer it owns: nothing is padded or copied per call, so such a plan runs in captured graphs like
+    any other, with the results of the eager run bit for bit, and no call allocates device memory."""
+    case = make_case(**BWD_CASES["head_dim_96"])
+    eager, ex = run_executor(case, backward=True)
+    check_against_truth(eager, dense_truth(case, backward=True))
+    graphed, _ = run_executor(case, backward=True, use_graph=True)
+    for a, b in zip(eager, graphed):
+        assert torch.equal(a.view(torch.int16) if a.dtype != torch.float32 else a.view(torch.int32),
+                           b.view(torch.int16) if b.dtype != torch.float32 else b.view(torch.int32))
+    # the prepared backward executes without allocating (the clones its API returns aside)
+    layout = case["layout"]
+    ex.execute(case["bw"], False)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    ex.execute(case["bw"], False)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+
+
 def test_forward_workspace_is_reusable_and_may_hold_anything(gpu):
     """The forward kernel hands out work items through counters in a caller workspace that each
     launch resets itself: a workspace full of garbage, reused by every attention launch of a
