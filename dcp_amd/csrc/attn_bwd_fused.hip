@@ -129,32 +129,48 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_prepare_kernel(const AttnBwdP
   const int o_slot = p.out_block_table[b];
   const int64_t row_stride = (int64_t)H * D;
   const int sub_lane = lane % LPP;
-  for (int pair0 = wave * PPW; pair0 < n_q * H; pair0 += (kBwdThreads / 64) * PPW) {
-    const int pair = pair0 + lane / LPP;
-    const bool live = pair < n_q * H;
-    const int ql = live ? pair / H : 0, head = live ? pair - ql * H : 0;
-    const int q_local = qt * kBwdBM + ql;
-    const int64_t off = (int64_t)o_slot * p.out_slot_stride + (int64_t)q_local * row_stride + (int64_t)head * D + sub_lane * 8;
-    const u32x4 o = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.out) + off);
-    const u32x4 g = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.dout) + off);
-    float dot = 0.0f;
+  // (four positions per round, all their words requested before anything is stored: the stores could
+  // alias the loads as far as the compiler knows, so it would not move a load above one itself)
+  constexpr int U = 4;
+  constexpr int STEP = (kBwdThreads / 64) * PPW;
+  for (int pair0 = wave * PPW; pair0 < n_q * H; pair0 += U * STEP) {
+    u32x4 o[U], g[U];
+    float l[U];
+    bool live[U];
+    int q_local[U], head[U];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      dot += Elem<DTYPE>::load((uint16_t)(o[i] & 0xffffu)) * Elem<DTYPE>::load((uint16_t)(g[i] & 0xffffu));
-      dot += Elem<DTYPE>::load((uint16_t)(o[i] >> 16)) * Elem<DTYPE>::load((uint16_t)(g[i] >> 16));
+    for (int u = 0; u < U; ++u) {
+      const int pair = pair0 + u * STEP + lane / LPP;
+      live[u] = pair < n_q * H;
+      const int ql = live[u] ? pair / H : 0;
+      head[u] = live[u] ? pair - ql * H : 0;
+      q_local[u] = qt * kBwdBM + ql;
+      const int64_t off = (int64_t)o_slot * p.out_slot_stride + (int64_t)q_local[u] * row_stride + (int64_t)head[u] * D + sub_lane * 8;
+      o[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.out) + off));  // read here only
+      g[u] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.dout) + off);
+      l[u] = p.lse[(int64_t)head[u] * p.lse_head_stride + (int64_t)o_slot * p.lse_slot_stride + q_local[u]];
     }
 #pragma unroll
-    for (int m = 1; m < LPP; m *= 2) dot += __shfl_xor(dot, m);
-    if (live && sub_lane == 0) {
-      const int64_t qrow = (int64_t)(q_begin + q_local) * H + head;
-      p.delta[qrow] = -dot;
-      p.lse2[qrow] = p.lse[(int64_t)head * p.lse_head_stride + (int64_t)o_slot * p.lse_slot_stride + q_local] * kLog2e;
-    }
-    if (nobody_visits && live) {  // no key tile sees these queries: their dQ is zero, and nobody else writes it
-      const u32x4 zero = {0, 0, 0, 0};
-      *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dq) +
-                                (int64_t)p.dq_block_table[b] * p.dq_slot_stride + (int64_t)q_local * row_stride + (int64_t)head * D +
-                                sub_lane * 8) = zero;
+    for (int u = 0; u < U; ++u) {
+      float dot = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        dot += Elem<DTYPE>::load((uint16_t)(o[u][i] & 0xffffu)) * Elem<DTYPE>::load((uint16_t)(g[u][i] & 0xffffu));
+        dot += Elem<DTYPE>::load((uint16_t)(o[u][i] >> 16)) * Elem<DTYPE>::load((uint16_t)(g[u][i] >> 16));
+      }
+#pragma unroll
+      for (int m = 1; m < LPP; m *= 2) dot += __shfl_xor(dot, m);
+      if (live[u] && sub_lane == 0) {
+        const int64_t qrow = (int64_t)(q_begin + q_local[u]) * H + head[u];
+        p.delta[qrow] = -dot;
+        p.lse2[qrow] = l[u] * kLog2e;
+      }
+      if (nobody_visits && live[u]) {  // no key tile sees these queries: their dQ is zero, and nobody else writes it
+        const u32x4 zero = {0, 0, 0, 0};
+        *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p.dq) +
+                                  (int64_t)p.dq_block_table[b] * p.dq_slot_stride + (int64_t)q_local[u] * row_stride +
+                                  (int64_t)head[u] * D + sub_lane * 8) = zero;
+      }
     }
   }
 }

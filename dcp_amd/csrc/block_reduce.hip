@@ -500,12 +500,14 @@ static int launch_merge(const void* src_out, void* dst_out, const float* src_lse
                    out_token_stride % VN == 0 &&
                    ((reinterpret_cast<uintptr_t>(src_out) | reinterpret_cast<uintptr_t>(dst_out)) &
                     15) == 0;
-  // the row-streaming kernel, when rows are dense over the heads, wide enough to give every lane of
-  // its workgroups work (a head block of 4 x 128 bf16 is not: 0.48 ms against 0.20 for the
-  // single-source merge of the 65536-token benchmark step) and the weights fit in LDS
-  if (vec && out_token_stride == (int64_t)n_head * head_dim && lse_token_stride == 1 &&
-      (int64_t)n_head * head_dim / VN * kRowTokens >= kMergeThreads * kRowUnroll &&
-      (int64_t)max_n_blocks_per_op * n_head * kRowTokens <= kRowWeightFloats) {
+  const bool dense_rows = vec && out_token_stride == (int64_t)n_head * head_dim && lse_token_stride == 1;
+  const bool wide = (int64_t)n_head * head_dim / VN * kRowTokens >= kMergeThreads * kRowUnroll &&
+                    (int64_t)max_n_blocks_per_op * n_head * kRowTokens <= kRowWeightFloats;
+  // the row-streaming kernels, when rows are dense over the heads, wide enough to give every lane of
+  // its workgroups work (a head block of 4 x 128 bf16 is not: the two-source merges of a 98304-token
+  // plan with two partials per row take 1.12 ms per step with the one-wave kernel against 0.50 with
+  // the lane-group kernel below) and the weights fit in LDS
+  if (dense_rows && wide) {
     const int wph = head_dim / VN, row_words = n_head * wph;
     if (max_n_blocks_per_op <= 4 && wph <= 64 && 64 % wph == 0 && wph % 4 == 0 && row_words % 64 == 0) {
       const int pieces_per_row = row_words / 64;
