@@ -29,7 +29,8 @@
 // takes 3.2 ms, 5.5 TB/s out of HBM, against 3.4 ms for four-wave workgroups with two stages and
 // a full wait per tile; a kernel that only streams 4 KiB pieces per wave into LDS the same way
 // reads 7.0 TB/s, and what is left between the two is the start of every work item (a chain of
-// dependent table reads and an empty pipeline, about 35 times per workgroup).
+// dependent table reads and an empty pipeline, about 35 times per workgroup: with no tiles at all
+// the kernel takes 0.21 ms, 6 us per item, and every item waits once for its first tile).
 #include <math.h>
 
 #include <algorithm>
