@@ -69,9 +69,15 @@ def _run(lib, pr, static):
     if static:
         _lib.call("dcp_attn_bwd_static", *head, *tail)
     else:
-        need = lib.dcp_attn_bwd_workspace_bytes(pr["n_rows"], pr["total_q"], pr["bs"], pr["hq"], pr["d"])
-        ws = torch.empty(need, dtype=torch.uint8, device=gpu)
-        _lib.call("dcp_attn_bwd", *head, ws.data_ptr(), need, *tail)
+        # the static entry point runs the two kernels that recompute: compare with the same backward,
+        # whichever one the process has selected for its other calls
+        before = lib.dcp_attn_bwd_select(0)
+        try:
+            need = lib.dcp_attn_bwd_workspace_bytes(pr["n_rows"], pr["total_q"], pr["bs"], pr["hq"], pr["d"])
+            ws = torch.empty(need, dtype=torch.uint8, device=gpu)
+            _lib.call("dcp_attn_bwd", *head, ws.data_ptr(), need, *tail)
+        finally:
+            lib.dcp_attn_bwd_select(before)
     torch.cuda.synchronize()
     return dq.view(torch.int16).cpu().numpy(), dkv.view(torch.int16).cpu().numpy()
 
