@@ -21,16 +21,19 @@
 // waves as in the other kernels.
 //
 // The kernel does nothing but wait for memory unless loads are in flight all the time (with the
-// matrix instructions taken out it runs as long as with them, and with the K loads or the barriers
-// taken out too), so a workgroup is eight waves (256 queries, one workgroup per CU: half the K traffic
-// of four-wave workgroups) with three stages of K tile and pieces in LDS: while tile t is multiplied,
-// the loads of tiles t + 1 and t + 2 are under way, and a wave waits for tile t alone by counting
-// its own loads (vmcnt), not for everything.  On the 65536-token causal benchmark (16.8 GB of dS) it
-// takes 3.2 ms, 5.5 TB/s out of HBM, against 3.4 ms for four-wave workgroups with two stages and
-// a full wait per tile; a kernel that only streams 4 KiB pieces per wave into LDS the same way
-// reads 7.0 TB/s, and what is left between the two is the start of every work item (a chain of
-// dependent table reads and an empty pipeline, about 35 times per workgroup: with no tiles at all
-// the kernel takes 0.21 ms, 6 us per item, and every item waits once for its first tile).
+// matrix instructions taken out it runs as long as with them), so a workgroup is eight waves (256
+// queries, one workgroup per CU: half the K traffic of four-wave workgroups) with three stages of
+// pieces in LDS: while step s is multiplied, the loads of steps s + 1 and s + 2 are under way, and a
+// wave waits for step s alone by counting its own loads (vmcnt), not for everything.  Where the kv
+// head has an even number of q heads a work item takes two of them, alternating between them tile
+// by tile: a K tile in LDS serves both heads' pieces (half the K loads again), and the waves meet at
+// a barrier only where the K tile changes, every other step.  On the 65536-token causal benchmark
+// (16.8 GB of dS) the kernel takes 3.0 ms, 5.9 TB/s out of HBM; with one head per item 3.2 ms;
+// with four-wave workgroups, two stages and a full wait per tile 3.4 ms.  A kernel that only
+// streams 4 KiB pieces per wave into LDS the same way reads 7.0 TB/s (6.6 with a workgroup barrier
+// per step, 6.0-6.2 with a K tile's loads beside it); the rest is the start of every work item (a
+// chain of dependent table reads and an empty pipeline: with no tiles at all the kernel takes
+// 0.21 ms, and every item waits once for its first tile).
 #include <math.h>
 
 #include <algorithm>
@@ -45,12 +48,17 @@ constexpr int kDsBM = 32 * kDsWaves;  // queries per workgroup
 constexpr int kDsBN = 64;             // keys per tile
 constexpr int kDsStages = 3;
 
-template <int DTYPE, int D>
+// HH: q heads per work item (1, or 2 of the same kv head).  With two, a K tile brought into LDS
+// serves both heads' pieces: the sequence of steps is (tile 0, head 0), (tile 0, head 1), (tile 1,
+// head 0), ... -- half the K loads, and a barrier only where the K tile changes (the pieces are
+// private to their wave).
+template <int DTYPE, int D, int HH>
 __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, int item) {
   constexpr int BN = kDsBN;
   constexpr int DT = D / 32;
+  constexpr int KSTAGES = HH == 1 ? kDsStages : 2;  // K tiles requested two steps ahead: two tiles, or one
   typedef KvTile<D, kDsWaves> Tile;
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[kDsStages][Tile::SIZE];
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[KSTAGES][Tile::SIZE];
   __shared__ __attribute__((aligned(16))) uint16_t ds_lds[kDsStages][kDsWaves][2048];  // [stage][wave]: one piece
   __shared__ int slot_lds[kSlotTableCap];
 
@@ -63,8 +71,8 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   int wg = item;
   const int qt = __builtin_amdgcn_readfirstlane(wg % p.dq_tiles_per_row);
   wg /= p.dq_tiles_per_row;
-  const int head = __builtin_amdgcn_readfirstlane(wg % p.n_heads_q);
-  const int bi = __builtin_amdgcn_readfirstlane(wg / p.n_heads_q);
+  const int head = __builtin_amdgcn_readfirstlane(wg % (p.n_heads_q / HH)) * HH;  // the item's first head
+  const int bi = __builtin_amdgcn_readfirstlane(wg / (p.n_heads_q / HH));
   const int b = __builtin_amdgcn_readfirstlane(p.row_order ? p.row_order[bi] : bi);
   const int q_begin = p.cu_seqlens_q[b];
   const int seqlen_q = p.cu_seqlens_q[b + 1] - q_begin;
@@ -114,11 +122,13 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   load_slot_table(slot_lds, kv_table, p.max_kv_blocks, tid, kDsThreads);
   __syncthreads();
 
-  f32x16 dq_acc[DT];
+  f32x16 dq_acc[HH][DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int hh = 0; hh < HH; ++hh)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) dq_acc[dt][i] = 0.0f;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dq_acc[hh][dt][i] = 0.0f;
 
   const uint16_t* kg = reinterpret_cast<const uint16_t*>(p.k) + (int64_t)kv_head * D;
   const uint32_t kv_goff0 = Tile::lane_offset0(p.kv_token_stride, w, lane);
@@ -139,18 +149,22 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
   const uint64_t piece0 = reinterpret_cast<uint64_t>(p.ds) +
                           ((row_base + ((uint64_t)head * p.subs_per_row + sub) * (uint64_t)last64) << 12);
   const uint64_t piece_step = 4096;
+  const uint64_t head_step = ((uint64_t)p.subs_per_row * (uint64_t)last64) << 12;  // to the next head's pieces
   auto wave_sees = [&](int t64) {
     const int t = t64 >> 1;
     return wave_has_tile && ((t >= mine.a0 && t < mine.b0) || (t >= mine.a1 && t < mine.b1));
   };
   constexpr int NL = Tile::LPW;
   uint32_t fill_k = 0, fill_ds = 0;
-  // everything tile `cursor` needs: this wave's share of the K tile, and its own piece if it sees the tile
-  auto request = [&]() {
+  // what a step needs: (for the item's first head) this wave's share of the K tile `cursor` points at,
+  // and the wave's own piece of that tile and head if it sees the tile
+  auto request = [&](int hh) {
+    if (hh == 0) {
 #pragma unroll
-    for (int i = 0; i < NL; ++i) Tile::load_group(fill_k, kg + cursor.off, kv_goff0, p.kv_token_stride, w, i);
+      for (int i = 0; i < NL; ++i) Tile::load_group(fill_k, kg + cursor.off, kv_goff0, p.kv_token_stride, w, i);
+    }
     if (wave_sees(cursor.tile)) {
-      const uint64_t src = uniform64(piece0 + (uint64_t)cursor.tile * piece_step);
+      const uint64_t src = uniform64(piece0 + hh * head_step + (uint64_t)cursor.tile * piece_step);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         Tile::load_group_at_streaming(__builtin_amdgcn_readfirstlane(fill_ds + i * 1024), uniform64(src + i * 1024), lane * 16);
@@ -160,7 +174,7 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
     if (cursor.index + 1 < n_tiles)
       cursor.advance(runs, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
   };
-  auto compute = [&](int t64, const uint16_t* k_lds, const uint16_t* piece) {
+  auto compute = [&](f32x16 (&acc)[DT], int t64, const uint16_t* k_lds, const uint16_t* piece) {
     if (!wave_sees(t64)) return;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -184,59 +198,84 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
         dsb[(ks + 1) & 1] = ds_operand(ks + 1);
       }
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) dq_acc[dt] = mfma_32x32x16<DTYPE>(kt_a[ks & 1][dt], dsb[ks & 1], dq_acc[dt]);
+      for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma_32x32x16<DTYPE>(kt_a[ks & 1][dt], dsb[ks & 1], acc[dt]);
     }
   };
 
-  // Stage s holds tile i with i % kDsStages == s.  Before it multiplies tile i, a wave waits until
-  // the loads it issued for tile i have landed -- the ones for tile i + 1, issued after them, may
-  // still be under way: vmcnt counts a wave's loads in order -- and meets the others at a barrier:
-  // everybody's share of K tile i is there, and everybody is done with tile i - 1, whose stage
-  // the loads of tile i + 2 now refill.
+  // Step s = (tile s / HH, head s % HH).  The pieces go through three stages (step s in stage
+  // s % 3), the K tiles through KSTAGES.  Before it multiplies step s, a wave waits until the loads it
+  // issued for step s have landed -- the ones for step s + 1, issued after them, may still be under
+  // way: vmcnt counts a wave's loads in order -- and, where the K tile changes, meets the others at a
+  // barrier: everybody's share of the K tile is there, and everybody is done with the tile before,
+  // whose stage (with three K stages: the stage of the tile before that) the loads of step s + 2
+  // now refill.  The pieces are private to their wave and need no barrier.
   const uint32_t k_at0 = lds_address(&k_lds[0][0]), ds_at0 = lds_address(&ds_lds[0][w][0]);
   constexpr uint32_t kKStageBytes = Tile::SIZE * 2, kDsStageBytes = kDsWaves * 4096;
-  auto request_into = [&](int stage) {
-    fill_k = k_at0 + stage * kKStageBytes;
-    fill_ds = ds_at0 + stage * kDsStageBytes;
-    request();
-  };
+  const int total = HH * n_tiles;
   if (n_tiles > 0) {
     cursor.seek(runs, 0, tiles_per_block, slot_lds, kv_table, p.kv_slot_stride, tile_stride);
-    request_into(0);
-    if (n_tiles > 1) {
-      advance();
-      request_into(1);
+    fill_k = k_at0;
+    fill_ds = ds_at0;
+    request(0);
+    if (total > 1) {
+      if (HH == 1) advance();
+      fill_k = k_at0 + kKStageBytes;  // (only used when this step brings a K tile: HH == 1)
+      fill_ds = ds_at0 + kDsStageBytes;
+      request(1 % HH);
     }
   }
-  int stage = 0;
-  for (int i = 0; i < n_tiles; ++i) {
-    if (i + 1 >= n_tiles) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else if (wave_sees(runs.tile(i + 1))) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL + 4) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
-    phase_barrier();
-    if (i + 2 < n_tiles) {
-      advance();
-      request_into(stage == 0 ? 2 : stage - 1);  // (i + 2) % 3
+  int ds_stage = 0, k_stage = 0;
+  for (int t = 0; t < n_tiles; ++t) {
+#pragma unroll
+    for (int hh = 0; hh < HH; ++hh) {
+      const int s_idx = t * HH + hh;
+      // the next step: its head, its tile, what it loads
+      const bool next_new_tile = hh + 1 == HH;
+      const int t_next = next_new_tile ? t + 1 : t;
+      if (s_idx + 1 >= total) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      } else {
+        const bool sees = wave_sees(runs.tile(t_next));
+        if (next_new_tile) {
+          if (sees) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL + 4) : "memory");
+          else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+        } else {
+          if (sees) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+      }
+      if (hh == 0) phase_barrier();
+      if (s_idx + 2 < total) {
+        // step s + 2: the same head as this one (HH is 1 or 2), tile t + 2 / HH
+        if (hh == 0) advance();
+        fill_ds = ds_at0 + (ds_stage == 0 ? 2 : ds_stage - 1) * kDsStageBytes;  // (s + 2) % 3
+        if (hh == 0) fill_k = k_at0 + (HH == 1 ? (k_stage == 0 ? 2 : k_stage - 1) : (k_stage ^ 1)) * kKStageBytes;
+        request(hh);
+      }
+      compute(dq_acc[hh], runs.tile(t), &k_lds[k_stage][0], &ds_lds[ds_stage][w][0]);
+      ds_stage = ds_stage == kDsStages - 1 ? 0 : ds_stage + 1;
     }
-    compute(runs.tile(i), &k_lds[stage][0], &ds_lds[stage][w][0]);
-    stage = stage == kDsStages - 1 ? 0 : stage + 1;
+    k_stage = k_stage == KSTAGES - 1 ? 0 : k_stage + 1;
   }
 
   if (!q_valid) return;
-  uint16_t* op = reinterpret_cast<uint16_t*>(p.dq) + (int64_t)p.dq_block_table[b] * p.dq_slot_stride +
-                 (int64_t)q_local * q_row_stride + (int64_t)head * D + 4 * h;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int hh = 0; hh < HH; ++hh) {
+    uint16_t* op = reinterpret_cast<uint16_t*>(p.dq) + (int64_t)p.dq_block_table[b] * p.dq_slot_stride +
+                   (int64_t)q_local * q_row_stride + (int64_t)(head + hh) * D + 4 * h;
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      u32x2 pk = {pack2<DTYPE>(dq_acc[dt][4 * gq] * p.scale, dq_acc[dt][4 * gq + 1] * p.scale),
-                  pack2<DTYPE>(dq_acc[dt][4 * gq + 2] * p.scale, dq_acc[dt][4 * gq + 3] * p.scale)};
-      *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * gq) = pk;
-    }
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        u32x2 pk = {pack2<DTYPE>(dq_acc[hh][dt][4 * gq] * p.scale, dq_acc[hh][dt][4 * gq + 1] * p.scale),
+                    pack2<DTYPE>(dq_acc[hh][dt][4 * gq + 2] * p.scale, dq_acc[hh][dt][4 * gq + 3] * p.scale)};
+        *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * gq) = pk;
+      }
+  }
 }
 
 // persistent, like the recomputing dQ kernel: per-XCD tickets in the workspace (zeroed by the prepare kernel)
-template <int DTYPE, int D>
+template <int DTYPE, int D, int HH>
 __global__ __launch_bounds__(kDsThreads, 1) void attn_bwd_dq_ds_kernel(const AttnBwdParams p) {
   __shared__ int ticket_lds;
   const int x = blockIdx.x % kNumXcd;
@@ -248,7 +287,7 @@ __global__ __launch_bounds__(kDsThreads, 1) void attn_bwd_dq_ds_kernel(const Att
     const int i = __builtin_amdgcn_readfirstlane(ticket_lds);
     if (i >= n_x) break;
     const int64_t item = (x + kNumXcd * (int64_t)(i / p.dq_xcd_group)) * p.dq_xcd_group + i % p.dq_xcd_group;
-    if (item < p.n_dq_items) attn_bwd_dq_ds_item<DTYPE, D>(fresh_kernel_args<AttnBwdParams>(), (int)item);
+    if (item < p.n_dq_items) attn_bwd_dq_ds_item<DTYPE, D, HH>(fresh_kernel_args<AttnBwdParams>(), (int)item);
     __syncthreads();
   }
 }
@@ -263,22 +302,27 @@ size_t bwd_ds_workspace_bytes(int64_t total_kv, int batch, int block_size, int n
 int launch_bwd_through_ds(const AttnBwdParams& p, int dtype, hipStream_t stream) {
   if (const int e = launch_bwd_prepare(p, dtype, stream)) return e;  // (also zeroes the dQ kernel's tickets)
   if (const int e = launch_bwd_dkv_writing_ds(p, dtype, stream)) return e;
-  // this dQ kernel's work items: (row, head, 256-query tile); the tiles and heads that share a K stay on one XCD
+  // this dQ kernel's work items: (row, one or two q heads of a kv head, 256-query tile); the tiles and
+  // heads that share a K stay on one XCD
+  const int per_kv = p.n_heads_q / p.n_heads_kv;
+  const int hh = per_kv % 2 == 0 ? 2 : 1;
   AttnBwdParams q = p;
   q.dq_tiles_per_row = (p.block_size + kDsBM - 1) / kDsBM;
-  q.n_dq_items = (int64_t)p.batch * p.n_heads_q * q.dq_tiles_per_row;
-  q.dq_xcd_group = q.dq_tiles_per_row * (p.n_heads_q / p.n_heads_kv);
+  q.n_dq_items = (int64_t)p.batch * (p.n_heads_q / hh) * q.dq_tiles_per_row;
+  q.dq_xcd_group = q.dq_tiles_per_row * (per_kv / hh);
   DCP_REQUIRE(q.n_dq_items < ((int64_t)1 << 31), "attn_bwd: grid too large");
   const int64_t n_dq = std::min<int64_t>(xcd_grid_size(q.n_dq_items, 1), xcd_grid_size((int64_t)device_cu_count(), 1));
   KernelTimer timer("attn_bwd_dq_ds_kernel", stream);
   const dim3 grid((unsigned)n_dq), block(kDsThreads);
+#define DCP_DQ_DS_LAUNCH(DT, HD, HH) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DT, HD, HH>), grid, block, 0, stream, q)
   if (dtype == DCP_DTYPE_BF16) {
-    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_BF16, 128>), grid, block, 0, stream, q);
-    else hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_BF16, 64>), grid, block, 0, stream, q);
+    if (p.head_dim == 128) { if (hh == 2) DCP_DQ_DS_LAUNCH(DCP_DTYPE_BF16, 128, 2); else DCP_DQ_DS_LAUNCH(DCP_DTYPE_BF16, 128, 1); }
+    else { if (hh == 2) DCP_DQ_DS_LAUNCH(DCP_DTYPE_BF16, 64, 2); else DCP_DQ_DS_LAUNCH(DCP_DTYPE_BF16, 64, 1); }
   } else {
-    if (p.head_dim == 128) hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_FP16, 128>), grid, block, 0, stream, q);
-    else hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<DCP_DTYPE_FP16, 64>), grid, block, 0, stream, q);
+    if (p.head_dim == 128) { if (hh == 2) DCP_DQ_DS_LAUNCH(DCP_DTYPE_FP16, 128, 2); else DCP_DQ_DS_LAUNCH(DCP_DTYPE_FP16, 128, 1); }
+    else { if (hh == 2) DCP_DQ_DS_LAUNCH(DCP_DTYPE_FP16, 64, 2); else DCP_DQ_DS_LAUNCH(DCP_DTYPE_FP16, 64, 1); }
   }
+#undef DCP_DQ_DS_LAUNCH
   return check_launch("attn_bwd_dq_ds_kernel");
 }
 
