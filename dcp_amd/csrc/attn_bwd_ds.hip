@@ -246,11 +246,12 @@ __device__ __forceinline__ void attn_bwd_dq_ds_item(KernArgs<AttnBwdParams>& p, 
       }
       if (hh == 0) phase_barrier();
       if (s_idx + 2 < total) {
-        // step s + 2: the same head as this one (HH is 1 or 2), tile t + 2 / HH
-        if (hh == 0) advance();
+        // step s + 2: head (hh + 2) % HH; it brings the next K tile along if that is the item's first head
+        const int hh_req = (hh + 2) % HH;  // (a constant once the loop over hh is unrolled)
+        if (hh_req == 0) advance();
         fill_ds = ds_at0 + (ds_stage == 0 ? 2 : ds_stage - 1) * kDsStageBytes;  // (s + 2) % 3
-        if (hh == 0) fill_k = k_at0 + (HH == 1 ? (k_stage == 0 ? 2 : k_stage - 1) : (k_stage ^ 1)) * kKStageBytes;
-        request(hh);
+        if (hh_req == 0) fill_k = k_at0 + (HH == 1 ? (k_stage == 0 ? 2 : k_stage - 1) : (k_stage ^ 1)) * kKStageBytes;
+        request(hh_req);
       }
       compute(dq_acc[hh], runs.tile(t), &k_lds[k_stage][0], &ds_lds[ds_stage][w][0]);
       ds_stage = ds_stage == kDsStages - 1 ? 0 : ds_stage + 1;
@@ -305,7 +306,7 @@ int launch_bwd_through_ds(const AttnBwdParams& p, int dtype, hipStream_t stream)
   // this dQ kernel's work items: (row, one or two q heads of a kv head, 256-query tile); the tiles and
   // heads that share a K stay on one XCD
   const int per_kv = p.n_heads_q / p.n_heads_kv;
-  const int hh = per_kv % 2 == 0 ? 2 : 1;
+  const int hh = per_kv % 2 == 0 ? 2 : 1;  // (four heads' accumulators do not fit the 256 registers of a wave)
   AttnBwdParams q = p;
   q.dq_tiles_per_row = (p.block_size + kDsBM - 1) / kDsBM;
   q.n_dq_items = (int64_t)p.batch * (p.n_heads_q / hh) * q.dq_tiles_per_row;
