@@ -63,6 +63,26 @@ def test_argument_errors_are_reported_without_a_launch(lib):
     assert lib.dcp_attn_bwd_workspace_bytes(2, 128, 64, 4, 128) >= 128 * 4 * 4 + 2 * 8 * 4
 
 
+def test_backward_selection_and_its_workspace_size(lib):
+    """dcp_attn_bwd_select returns the previous setting and only sets a known mode; the workspace the
+    selected backward needs: the recomputing one the small scratch whatever the key count, the one
+    that keeps dS in memory 4 KiB per (64-key tile, head, 32-query chunk) on top of it, with one tile
+    more per row than total_kv / 64 and two spare pieces."""
+    before = lib.dcp_attn_bwd_select(0)
+    try:
+        assert lib.dcp_attn_bwd_select(-1) == 0 and lib.dcp_attn_bwd_select(77) == 0 and lib.dcp_attn_bwd_select(-1) == 0
+        batch, total_q, total_kv, bs, heads, d = 6, 6 * 256, 6 * 1024 + 5 * 256, 256, 4, 128
+        base = lib.dcp_attn_bwd_workspace_bytes(batch, total_q, bs, heads, d)
+        assert lib.dcp_attn_bwd_workspace_bytes_kv(batch, total_q, total_kv, bs, heads, d) == base
+        assert lib.dcp_attn_bwd_select(2) == 0
+        pieces = (total_kv // 64 + batch + 1) * heads * (bs // 32) + 2
+        assert lib.dcp_attn_bwd_workspace_bytes_kv(batch, total_q, total_kv, bs, heads, d) == base + pieces * 4096
+        assert lib.dcp_attn_bwd_workspace_bytes_kv(batch, total_q, 0, bs, heads, d) == base, "no key count: nothing to keep"
+        assert lib.dcp_attn_bwd_workspace_bytes(batch, total_q, bs, heads, d) == base
+    finally:
+        lib.dcp_attn_bwd_select(before)
+
+
 def test_profile_report_is_empty_when_disabled(lib):
     from dcp_amd import _lib
 
