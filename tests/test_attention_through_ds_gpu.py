@@ -24,6 +24,10 @@ CASES = {
     "shared_question_fp16": dict(seqlens=[700], block_size=128, n_heads=2, n_groups=1, head_dim=128, head_block=2,
                                  mask="shared_question", mask_kwargs=dict(question_proportion=0.3, n_answers=3),
                                  dtype="fp16", qkv_scale=0.5),
+    # three q heads per kv head (the dQ kernel takes two heads per work item only where their number is even),
+    # 320-token blocks (a 256-query work item and a ragged second one)
+    "three_heads_per_kv_head": dict(seqlens=[700, 100], block_size=320, n_heads=6, n_groups=2, head_dim=128, head_block=3,
+                                    qkv_scale=0.5),
     # 64-token blocks, key counts below and just above one 64-key piece
     "tiny_blocks": dict(seqlens=[70, 33, 5], block_size=64, n_heads=2, n_groups=1, head_dim=128, head_block=2,
                         qkv_scale=0.5),
